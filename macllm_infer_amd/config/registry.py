@@ -1,6 +1,6 @@
 """One registry from an architecture's name to its configuration class.
 
-``config.json`` names its architecture in ``architectures[0]`` (or ``model_type``);
+``config.json`` names its architecture in ``architectures[0]`` (or ``model_type``, or ``architecture``);
 the class registered under that name reads the rest of the file and lowers it to a
 ``ModelSpec``.  The reference resolves a file the same way: architecture string ->
 spec builder -> adapter (src/gguf_model.rs:315-354, :391-444), and an unknown name is
@@ -36,10 +36,11 @@ def config_from_dict(raw: dict):
     architectures = raw.get("architectures")
     if isinstance(architectures, list) and architectures:
         names.append(architectures[0])
-    if isinstance(raw.get("model_type"), str):
-        names.append(raw["model_type"])
+    for key in ("model_type", "architecture"):
+        if isinstance(raw.get(key), str):
+            names.append(raw[key])
     if not names:
-        raise ConfigError("config.json names no architecture ('architectures' or 'model_type'); "
+        raise ConfigError("config.json names no architecture ('architectures', 'model_type' or 'architecture'); "
                           f"registered: {registered_architectures()}")
     for name in names:
         if name in _ARCHITECTURES:

@@ -52,11 +52,24 @@ class NoPositionSpec:
 
 @dataclass(frozen=True)
 class RmsNormSpec:
+    """``weight_offset``: what is added to the stored weight (1.0 for a weight stored around zero)."""
     eps: float
+    weight_offset: float = 0.0
     kind: str = "rmsnorm"
 
     def validate(self) -> None:
         _require(self.eps > 0, f"norm eps must be positive, got {self.eps}")
+
+
+@dataclass(frozen=True)
+class LogDistanceBiasSpec:
+    """No rotation; the score of a key at distance n behind the query loses r1 * ln(1 + r2 * n), with r1 and
+    r2 learned numbers of each query head (tensors ``r1`` and ``r2`` of the mixer)."""
+    num_heads: int
+    kind: str = "log_distance"
+
+    def validate(self, head_dim: int) -> None:
+        _require(self.num_heads > 0, "a distance bias needs the number of query heads")
 
 
 @dataclass(frozen=True)
@@ -65,6 +78,8 @@ class AttentionSpec:
 
     ``window``: None = every earlier key; w = the w most recent keys, the query's own
     included (a key is masked when query - key >= w, src/decoder.rs:4521-4526).
+    ``value_dim``: values may be narrower or wider than keys.  ``sink``: a learned number per query
+    head that takes part in the softmax's denominator without a key or a value.
     Multipliers scale the normed input, the key projection's output and the output
     projection's output.
     """
@@ -79,11 +94,18 @@ class AttentionSpec:
     in_multiplier: float = 1.0
     key_multiplier: float = 1.0
     out_multiplier: float = 1.0
+    value_dim: Optional[int] = None      # width of a value head (None: the keys' head_dim)
+    sink: bool = False                   # one more term exp(sink[head]) in the softmax's denominator (tensor ``sink``)
     kind: str = "attention"
+
+    @property
+    def value_width(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
     def validate(self) -> None:
         _require(self.num_heads > 0 and self.num_kv_heads > 0,
                  "attention head counts must be positive")
+        _require(self.value_width > 0, "the width of a value head must be positive")
         _require(self.num_heads % self.num_kv_heads == 0,
                  f"num_attention_heads {self.num_heads} is not a multiple of "
                  f"num_key_value_heads {self.num_kv_heads}")
@@ -138,6 +160,63 @@ class Mamba2Spec:
 
 
 @dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head and no softmax: S <- decay[h] S + k v^T, o = S^T q, the
+    state [key_dim, value_dim] per head carried in float32.  q and k are turned by ``position`` (a rotation of the
+    first dims of a head, or none), k is then multiplied by ``key_scale``; each head's o is divided by its root
+    mean square (``norm_eps``), gated by SiLU of a fourth projection and projected out."""
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay: Tuple[float, ...]
+    key_scale: float
+    norm_eps: float
+    position: object = field(default_factory=NoPositionSpec)
+    kind: str = "retention"
+
+    def validate(self) -> None:
+        _require(self.num_heads > 0 and self.key_dim > 0 and self.value_dim > 0, "retention sizes must be positive")
+        _require(len(self.decay) == self.num_heads,
+                 f"retention needs one decay per head: {len(self.decay)} given for {self.num_heads} heads")
+        _require(all(d == d and abs(d) != float("inf") for d in self.decay), "retention decays must be finite")
+        _require(self.norm_eps > 0, "retention norm eps must be positive")
+        self.position.validate(self.key_dim)
+
+
+@dataclass(frozen=True)
+class GeneralDeltaSpec:
+    """Generalized delta rule: per head a state S [dim, dim] in float32 with
+    S <- diag(w) S - (a * u)(u^T S) + k v^T (u the unit key, both products on the old state), o = S^T r.
+    w = exp(-``decay_floor`` * sigmoid(w2 tanh(w1 h) + w0)) per head and key channel, a = sigmoid(a h + bias).
+    ``decay_rank``: the inner width of the decay's two projections (None: whatever the stored tensors have)."""
+    num_heads: int
+    head_dim: int
+    norm_eps: float
+    decay_floor: float = 0.6065306597126334     # exp(-1/2)
+    key_eps: float = 1e-6                        # inside the root of the unit key
+    decay_rank: Optional[int] = None
+    kind: str = "general_delta"
+
+    def validate(self) -> None:
+        _require(self.num_heads > 0 and self.head_dim > 0, "general_delta sizes must be positive")
+        _require(self.decay_rank is None or self.decay_rank > 0, "general_delta decay_rank must be positive")
+        _require(self.norm_eps > 0 and self.key_eps > 0, "general_delta eps must be positive")
+
+
+@dataclass(frozen=True)
+class PolyNormFFNSpec:
+    """down(act(up(x))) with act(z) = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers element by element, N the
+    division of a token's row by its root mean square (``eps``); the four numbers are the tensor ``act``."""
+    intermediate_size: int
+    eps: float
+    kind: str = "polynorm_ffn"
+
+    def validate(self) -> None:
+        _require(self.intermediate_size > 0, "the feed-forward width must be positive")
+        _require(self.eps > 0, "the feed-forward's norm eps must be positive")
+
+
+@dataclass(frozen=True)
 class SwiGLUSpec:
     """down(SiLU(gate(x) * gate_multiplier) * up(x)) * down_multiplier (src/decoder.rs:261-306)."""
     intermediate_size: int
@@ -165,7 +244,8 @@ class LayerSpec:
     h += ffn(norm(h)) (src/decoder.rs:2658-2699).  One mixer gives the ordinary
     sequential pre-norm layer.  ``prefix`` is the tensor-name path of the layer;
     ``mixer_norm_name`` / ``ffn_norm_name`` / ``ffn_name`` the sub-paths below it
-    (src/architecture.rs:1543-1567, :1639-1647).
+    (src/architecture.rs:1543-1567, :1639-1647).  ``ffn`` None: the layer is its mixers alone (a checkpoint may
+    still hold the second norm and scale of such a layer; they are not used).
     """
     prefix: str
     mixers: Tuple[MixerSlot, ...]
@@ -176,6 +256,10 @@ class LayerSpec:
     ffn_norm_name: str = "ffn_norm"
     ffn_name: str = "mlp"
     arrangement: str = "parallel_prenorm"
+    # tensors [hidden] that multiply the mixers' summed output / the feed-forward's output, feature by feature,
+    # before it is added to the residual stream (None: no such scale)
+    mixer_scale_name: Optional[str] = None
+    ffn_scale_name: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -210,8 +294,18 @@ class ModelSpec:
     tensor_aliases: Tuple[Tuple[str, str], ...] = ()
     # a checkpoint none of whose names starts with this gets it in front of all but the output head's
     root_namespace: str = "model."
+    # (regular expression, replacement) pairs that turn a tensor's name in the model into the name the
+    # architecture's checkpoints store it under, applied in order (``stored_name``)
+    stored_name_rules: Tuple[Tuple[str, str], ...] = ()
     # ("part kind.spec field", the configuration file's key for it): for messages that name a field
     field_names: Tuple[Tuple[str, str], ...] = ()
+
+    def stored_name(self, name: str) -> str:
+        """The name under which the architecture's checkpoints hold the model's tensor ``name``."""
+        import re
+        for pattern, replacement in self.stored_name_rules:
+            name = re.sub(pattern, replacement, name)
+        return name
 
     def validate(self) -> None:
         """Positivity, divisibility and bounds, field by field (src/architecture.rs:367-452)."""
@@ -230,9 +324,10 @@ class ModelSpec:
             _require(len(set(names)) == len(names), f"layer {layer.prefix} names a mixer twice")
             for slot in layer.mixers:
                 slot.spec.validate()
-            layer.ffn.validate()
             layer.mixer_norm.validate()
-            layer.ffn_norm.validate()
+            if layer.ffn is not None:
+                layer.ffn.validate()
+                layer.ffn_norm.validate()
         for index, entry in enumerate(self.schedule):
             _require(0 <= entry.layer < len(self.layers),
                      f"schedule entry {index} names layer {entry.layer}, which does not exist")

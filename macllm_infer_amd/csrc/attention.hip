@@ -7,7 +7,8 @@
 // contiguous.  Entry points get the base pointers of one layer's K and V inside page 0 and
 // the stride between pages:
 //   K(page, kvh, off, i) = k_base + page*page_stride + (kvh*page_size + off)*dh + i
-//   V(page, kvh, off, i) = v_base + page*page_stride + (kvh*dh + i)*page_size + off
+//   V(page, kvh, off, i) = v_base + page*page_stride + (kvh*dv + i)*page_size + off
+// with dv the width of a value head, which the general kernels take apart from dh, the width of a key head.
 // (The reference pages its cache the same way, K and V both token-major:
 // crates/macllm-kv/src/cache.rs:558-566, crates/macllm-kernels/src/metal/paged_decode.metal:109-113.)
 #include "common.h"
@@ -21,7 +22,7 @@
 //   (reference: src/decoder.rs:186-195, 226-229; K is cached after rotation, :953-962)
 // slot_mapping[t] = page*page_size + offset of the token's cache cell; null = nothing is stored.
 template <typename T>
-__global__ void rope_kv_store_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh,
+__global__ void rope_kv_store_kernel(T* __restrict__ qkv, long ld, int Hq, int Hkv, int dh, int dv,
                                      const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                      int rotary_dim, const int* __restrict__ slot_mapping,
                                      T* __restrict__ k_base, T* __restrict__ v_base, long page_stride,
@@ -82,29 +83,30 @@ __global__ void rope_kv_store_kernel(T* __restrict__ qkv, long ld, int Hq, int H
   }
   if (cell >= 0) {
     const T* v = row + (long)(Hq + Hkv) * dh;
-    for (int item = threadIdx.x; item < Hkv * dh; item += blockDim.x) {
-      const int kvh = item / dh;
-      const int i = item - kvh * dh;
-      v_base[page * page_stride + ((long)kvh * dh + i) * page_size + offset] = v[item];
+    for (int item = threadIdx.x; item < Hkv * dv; item += blockDim.x) {
+      const int kvh = item / dv;
+      const int i = item - kvh * dv;
+      v_base[page * page_stride + ((long)kvh * dv + i) * page_size + offset] = v[item];
     }
   }
 }
 
-extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, int Hkv, int dh,
+// dv: the width of a value head (the v heads follow the k heads in a row of qkv).
+extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, int Hkv, int dh, int dv,
                                 const int* positions, const float* inv_freq, int rotary_dim,
                                 const int* slot_mapping, void* k_base, void* v_base, long page_stride,
                                 int page_size, hipStream_t stream) {
-  if (T <= 0 || Hq <= 0 || Hkv <= 0 || dh <= 0 || (dh & 1)) return ERR_BAD_ARGUMENT;
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || dh <= 0 || (dh & 1) || dv <= 0) return ERR_BAD_ARGUMENT;
   if (rotary_dim < 0 || rotary_dim > dh || (rotary_dim & 1)) return ERR_BAD_ARGUMENT;
-  if (ld < (long)(Hq + 2 * Hkv) * dh) return ERR_BAD_ARGUMENT;
+  if (ld < (long)(Hq + Hkv) * dh + (long)Hkv * dv) return ERR_BAD_ARGUMENT;
   if (slot_mapping && (!k_base || !v_base || page_size <= 0)) return ERR_BAD_ARGUMENT;
   if (!inv_freq) rotary_dim = 0;
   if (dtype == DT_F32)
-    rope_kv_store_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, ld, Hq, Hkv, dh, positions, inv_freq,
+    rope_kv_store_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, ld, Hq, Hkv, dh, dv, positions, inv_freq,
                                                         rotary_dim, slot_mapping, (float*)k_base,
                                                         (float*)v_base, page_stride, page_size);
   else if (dtype == DT_BF16)
-    rope_kv_store_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)qkv, ld, Hq, Hkv, dh, positions, inv_freq,
+    rope_kv_store_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)qkv, ld, Hq, Hkv, dh, dv, positions, inv_freq,
                                                          rotary_dim, slot_mapping, (bf16_t*)k_base,
                                                          (bf16_t*)v_base, page_stride, page_size);
   else
@@ -121,6 +123,11 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 //   softmax in float32 (reference: src/decoder.rs:4665-4667).
 // `slopes` (optional, float32 per query head): a position encoding that is a bias on the scores,
 //   s -= slopes[head] * (query position - key position)   (no counterpart in the reference).
+// `log_bias` (optional, float32 [query heads][2] = (r1, r2)): a bias that grows with the logarithm of the distance,
+//   s -= r1 * ln(1 + r2 * (query position - key position)).
+// `sinks` (optional, float32 per query head, read by the merge kernel): exp(sink) is one more term of the softmax's
+//   denominator; it has no key and no value.
+// dv: the width of a value head; the partial results and the output have dv dims a head.
 // The keys are cut into runs of PA_RUN by their absolute position.  One workgroup per (token, query head,
 // run): each of its four waves takes 64 keys of the run (lane i scores key i with a full dot product over
 // dh from its own cache row; for the value product lane i owns output dims i, i + 64, ...), keeps
@@ -135,15 +142,16 @@ extern "C" int mi_rope_kv_store(void* qkv, int dtype, long ld, int T, int Hq, in
 
 template <typename T, bool FAST_EXP>
 __global__ void __launch_bounds__(PA_RUN)
-paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh,
+paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh, int dv,
                        const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                        int page_size, const int* __restrict__ block_tables, int max_pages,
                        const int* __restrict__ lane_of_token, const int* __restrict__ positions, float scale,
-                       int window, const float* __restrict__ slopes, int runs, float* __restrict__ partial) {
+                       int window, const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
+                       float* __restrict__ partial) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
   __shared__ __align__(16) float q_shared[ATT_MAX_DH];
   __shared__ float p_shared[PA_WAVES][WAVE];
-  __shared__ long row_shared[PA_WAVES][WAVE];     // base of the key's (page, kv head) block
+  __shared__ long row_shared[PA_WAVES][WAVE];     // base of the key's (page, kv head) block of values
   __shared__ int offset_shared[PA_WAVES][WAVE];   // the key's place inside its page
   __shared__ float wave_ml[PA_WAVES][2];
   __shared__ float wave_o[PA_WAVES][ATT_MAX_DH];
@@ -171,8 +179,8 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   if (visible) {
     const int page = table[key / page_size];
     offset = key % page_size;
-    row_offset = (long)page * page_stride + (long)kvh * page_size * dh;
-    const T* k_row = k_base + row_offset + (long)offset * dh;
+    row_offset = (long)page * page_stride + (long)kvh * page_size * dv;
+    const T* k_row = k_base + (long)page * page_stride + ((long)kvh * page_size + offset) * dh;
     float dot = 0.f;
     if (dh % 4 == 0 && page_stride % 4 == 0 && ((unsigned long long)k_base % (4 * sizeof(T))) == 0) {
       for (int i = 0; i < dh; i += 4) {
@@ -185,6 +193,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
     }
     score = dot * scale;
     if (slopes) score = fmaf(-slopes[head], (float)(query_position - key), score);
+    if (log_bias) score = fmaf(-log_bias[2 * head], log1pf(log_bias[2 * head + 1] * (float)(query_position - key)), score);
   }
   const float maximum = wave_max(score);                    // -inf for a wave without visible keys
   const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
@@ -206,7 +215,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
 #pragma unroll
   for (int i = 0; i < ATT_MAX_DH / WAVE; ++i) {
     const int dim = lane + i * WAVE;
-    if (dim < dh) {
+    if (dim < dv) {
       // sixteen values asked for at once, then added in the order of their keys (one at a time, each load would
       // wait for the one before: 64 round trips a wave); a key past the last reads the last again and is not added
       float sum = 0.f;
@@ -232,7 +241,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
   float best = wave_ml[0][0];
 #pragma unroll
   for (int w = 1; w < PA_WAVES; ++w) best = fmaxf(best, wave_ml[w][0]);
-  float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dh + 2);
+  float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dv + 2);
   float weight[PA_WAVES];
   float denominator = 0.f;
 #pragma unroll
@@ -244,7 +253,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int 
     mine[0] = best;
     mine[1] = denominator;
   }
-  for (int dim = tid; dim < dh; dim += PA_RUN) {
+  for (int dim = tid; dim < dv; dim += PA_RUN) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < PA_WAVES; ++w) sum = fmaf(weight[w], wave_o[w][dim], sum);
@@ -288,12 +297,13 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
 // DIMS: dims of a head a lane sums (1, 2 or 4: the head size in units of 64, rounded up)
 template <typename T, bool FAST_EXP, int DIMS>
 __global__ void __launch_bounds__(PA_RUN)
-paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh,
+paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv, int dh, int dv,
                             const T* __restrict__ k_base, const T* __restrict__ v_base, long page_stride,
                             int page_size, const int* __restrict__ block_tables, int max_pages,
                             const int* __restrict__ query_tiles, int tile_tokens, const int* __restrict__ cu_seqlens,
                             const int* __restrict__ positions, float scale, int window,
-                            const float* __restrict__ slopes, int runs, float* __restrict__ partial) {
+                            const float* __restrict__ slopes, const float* __restrict__ log_bias, int runs,
+                            float* __restrict__ partial) {
   typedef T vec4 __attribute__((ext_vector_type(4)));
   extern __shared__ __align__(16) float tile_lds[];
   const int k_ld = dh + PT_PAD;                      // a key's row in LDS
@@ -301,8 +311,8 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
   const int p_ld = WAVE + PT_PAD;                    // a query's row of probabilities in LDS
   float* q_lds = tile_lds;                           // [PT_QUERIES][dh]
   float* k_lds = q_lds + PT_QUERIES * dh;            // [64][k_ld]
-  float* v_lds = k_lds + WAVE * k_ld;                // [dh][v_ld]
-  float* p_lds = v_lds + dh * v_ld;                  // [PA_WAVES][PT_PER_WAVE][p_ld]
+  float* v_lds = k_lds + WAVE * k_ld;                // [dv][v_ld]
+  float* p_lds = v_lds + dv * v_ld;                  // [PA_WAVES][PT_PER_WAVE][p_ld]
   const int subtiles = tile_tokens / PT_QUERIES;
   const int tile = blockIdx.x / subtiles;
   const int head = blockIdx.y;
@@ -381,10 +391,10 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       if (key_in < keys && key_in >= skipped) {
         const int key = group_first + key_in;
         const int page = table[key / page_size];
-        const T* from = v_base + (long)page * page_stride + (long)kvh * dh * page_size + key % page_size;
-        for (int dim = wave; dim < dh; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = to_float(from[(long)dim * page_size]);
+        const T* from = v_base + (long)page * page_stride + (long)kvh * dv * page_size + key % page_size;
+        for (int dim = wave; dim < dv; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = to_float(from[(long)dim * page_size]);
       } else {
-        for (int dim = wave; dim < dh; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = 0.f;
+        for (int dim = wave; dim < dv; dim += PA_WAVES) v_lds[dim * v_ld + key_in] = 0.f;
       }
     }
     __syncthreads();
@@ -421,6 +431,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       if (visible) {
         score = dot[i] * scale;
         if (slopes) score = fmaf(-slopes[head], (float)(position - key), score);
+        if (log_bias) score = fmaf(-log_bias[2 * head], log1pf(log_bias[2 * head + 1] * (float)(position - key)), score);
       }
       const float maximum = wave_max_dpp(score);
       const float p = visible ? (FAST_EXP ? __expf(score - maximum) : expf(score - maximum)) : 0.f;
@@ -439,7 +450,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
         for (int d = 0; d < DIMS; ++d) sums[i][d] = 0.f;
       const float* v_row[DIMS];
 #pragma unroll
-      for (int d = 0; d < DIMS; ++d) v_row[d] = v_lds + min(lane + d * WAVE, dh - 1) * v_ld;
+      for (int d = 0; d < DIMS; ++d) v_row[d] = v_lds + min(lane + d * WAVE, dv - 1) * v_ld;
       // the normalizers: lane i adds the probabilities of query i in the order of the keys
       const float* p_mine = p_rows + (lane & (PT_PER_WAVE - 1)) * p_ld;
       float normalizer = 0.f;
@@ -455,7 +466,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
         for (int i = 0; i < PT_PER_WAVE; ++i) pj[i] = *reinterpret_cast<const float4*>(p_rows + i * p_ld + j);
 #pragma unroll
         for (int d = 0; d < DIMS; ++d) {
-          if (d * WAVE < dh) {                          // the same for every lane
+          if (d * WAVE < dv) {                          // the same for every lane
             const float4 vj = *reinterpret_cast<const float4*>(v_row[d] + j);
 #pragma unroll
             for (int i = 0; i < PT_PER_WAVE; ++i) {
@@ -499,7 +510,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
       denominator = fmaf(weight[g], group_norm[i][g], denominator);
     }
     const long token = first_row + wave + i * PA_WAVES;
-    float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dh + 2);
+    float* mine = partial + ((token * Hq + head) * runs + run) * (long)(dv + 2);
     if (lane == 0) {
       mine[0] = best;
       mine[1] = denominator;
@@ -507,7 +518,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
 #pragma unroll
     for (int d = 0; d < DIMS; ++d) {
       const int dim = lane + d * WAVE;
-      if (dim < dh) {
+      if (dim < dv) {
         float sum = 0.f;
 #pragma unroll
         for (int g = 0; g < PA_WAVES; ++g) sum = fmaf(weight[g], group_o[i][g][d], sum);
@@ -520,7 +531,7 @@ paged_attention_tile_kernel(const T* __restrict__ q, long q_ld, int Hq, int Hkv,
 template <typename T, bool FAST_EXP>
 __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, int Hq, int dh, int runs,
                                              const int* __restrict__ positions, int window,
-                                             T* __restrict__ out, long out_ld) {
+                                             const float* __restrict__ sinks, T* __restrict__ out, long out_ld) {
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int query_position = positions[token];
@@ -542,6 +553,14 @@ __global__ void paged_attention_merge_kernel(const float* __restrict__ partial, 
       sum = sum * keep + weight * one[2 + dim];
       maximum = larger;
     }
+    if (sinks) {
+      // the sink: a term of the denominator that brings no value
+      const float sink = sinks[head];
+      const float larger = fmaxf(maximum, sink);
+      const float keep = FAST_EXP ? __expf(maximum - larger) : expf(maximum - larger);
+      denominator = denominator * keep + (FAST_EXP ? __expf(sink - larger) : expf(sink - larger));
+      sum *= keep;
+    }
     out[token * out_ld + (long)head * dh + dim] = from_float<T>(sum / denominator);
   }
 }
@@ -554,8 +573,8 @@ extern "C" long mi_paged_attention_workspace(int T, int Hq, int dh, int max_seq_
 }
 
 // LDS of a workgroup of the tiled kernel: the tile's queries, 64 keys, their values, a wave's probabilities
-static size_t paged_attention_tile_lds(int dh) {
-  return ((size_t)PT_QUERIES * dh + (size_t)WAVE * (dh + PT_PAD) + (size_t)dh * (WAVE + PT_PAD) +
+static size_t paged_attention_tile_lds(int dh, int dv) {
+  return ((size_t)PT_QUERIES * dh + (size_t)WAVE * (dh + PT_PAD) + (size_t)dv * (WAVE + PT_PAD) +
           (size_t)PT_QUERIES * (WAVE + PT_PAD)) * sizeof(float);
 }
 
@@ -578,63 +597,70 @@ static int raise_tile_lds(size_t bytes) {
 // query_tiles (optional) [num_tiles, 2] = (lane or -1, first token row) of runs of up to tile_tokens tokens of one
 // lane (tile_tokens a multiple of 16), with cu_seqlens [lanes + 1]: the step's lanes hold several tokens, and the
 // partial results come from the kernel that shares a run's keys among the queries of a tile (the same bits).
-extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh,
+// dv: the width of a value head (the work area is sized for it: mi_paged_attention_workspace(T, Hq, dv, ...));
+// log_bias, sinks: see above.
+extern "C" int mi_paged_attention(const void* q, int dtype, long q_ld, int T, int Hq, int Hkv, int dh, int dv,
                                   const void* k_base, const void* v_base, long page_stride, int page_size,
                                   const int* block_tables, int max_pages, const int* lane_of_token,
                                   const int* positions, float scale, int window, const float* slopes,
+                                  const float* log_bias, const float* sinks,
                                   int max_seq_len, float* partial, long partial_floats, void* out, long out_ld,
                                   const int* query_tiles, int num_tiles, int tile_tokens, const int* cu_seqlens,
                                   hipStream_t stream) {
-  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || page_size <= 0 || max_pages <= 0 ||
+  if (T <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || dh <= 0 || dv <= 0 || page_size <= 0 || max_pages <= 0 ||
       max_seq_len <= 0 || !partial)
     return ERR_BAD_ARGUMENT;
-  if (dh > ATT_MAX_DH) return ERR_UNSUPPORTED_SIZE;
+  if (dh > ATT_MAX_DH || dv > ATT_MAX_DH) return ERR_UNSUPPORTED_SIZE;
   const int runs = (max_seq_len + PA_RUN - 1) / PA_RUN;
   if (Hq > 65535 || runs > 65535) return ERR_UNSUPPORTED_SIZE;
-  if (partial_floats < mi_paged_attention_workspace(T, Hq, dh, max_seq_len)) return ERR_BAD_ARGUMENT;
+  if (partial_floats < mi_paged_attention_workspace(T, Hq, dv, max_seq_len)) return ERR_BAD_ARGUMENT;
   const int element = dtype == DT_F32 ? 4 : 2;
   // the tiled kernel: head sizes in steps of 16, 4 elements a load from the cache
   bool tiled = query_tiles != nullptr && num_tiles > 0 && cu_seqlens != nullptr && tile_tokens > 0 &&
                tile_tokens % PT_QUERIES == 0 && dh % 16 == 0 && page_stride % 4 == 0 &&
                ((uintptr_t)k_base % (4 * element)) == 0 && (long)num_tiles * (tile_tokens / PT_QUERIES) <= 0x7fffffffL;
-  const size_t tile_lds = paged_attention_tile_lds(dh);
-  const int dims = dh <= WAVE ? 1 : dh <= 2 * WAVE ? 2 : 4;
+  const size_t tile_lds = paged_attention_tile_lds(dh, dv);
+  const int dims = dv <= WAVE ? 1 : dv <= 2 * WAVE ? 2 : 4;
   if (tiled && tile_lds > 64 * 1024) {
     int code;
-    if (dtype == DT_F32) code = dims == 2 ? raise_tile_lds<float, false, 2>(tile_lds) : raise_tile_lds<float, false, 4>(tile_lds);
-    else code = dims == 2 ? raise_tile_lds<bf16_t, true, 2>(tile_lds) : raise_tile_lds<bf16_t, true, 4>(tile_lds);
+    if (dtype == DT_F32)
+      code = dims == 1 ? raise_tile_lds<float, false, 1>(tile_lds)
+                       : dims == 2 ? raise_tile_lds<float, false, 2>(tile_lds) : raise_tile_lds<float, false, 4>(tile_lds);
+    else
+      code = dims == 1 ? raise_tile_lds<bf16_t, true, 1>(tile_lds)
+                       : dims == 2 ? raise_tile_lds<bf16_t, true, 2>(tile_lds) : raise_tile_lds<bf16_t, true, 4>(tile_lds);
     if (code != 0) tiled = false;                      // the per-token kernel takes any size
   }
   const dim3 grid(T, Hq, runs);
   const dim3 tile_grid(tiled ? num_tiles * (tile_tokens / PT_QUERIES) : 1, Hq, runs);
   const dim3 merge_grid(T, Hq);
-  const int merge_threads = dh <= WAVE ? WAVE : dh <= 2 * WAVE ? 2 * WAVE : 4 * WAVE;
+  const int merge_threads = dv <= WAVE ? WAVE : dv <= 2 * WAVE ? 2 * WAVE : 4 * WAVE;
   if (dtype == DT_F32) {
 #define TILE_LAUNCH(T_, FAST_, DIMS_)                                                                                 \
   paged_attention_tile_kernel<T_, FAST_, DIMS_><<<tile_grid, PA_RUN, tile_lds, stream>>>(                              \
-      (const T_*)q, q_ld, Hq, Hkv, dh, (const T_*)k_base, (const T_*)v_base, page_stride, page_size, block_tables,     \
-      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, runs, partial)
+      (const T_*)q, q_ld, Hq, Hkv, dh, dv, (const T_*)k_base, (const T_*)v_base, page_stride, page_size, block_tables, \
+      max_pages, query_tiles, tile_tokens, cu_seqlens, positions, scale, window, slopes, log_bias, runs, partial)
     if (tiled && dims == 1) TILE_LAUNCH(float, false, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(float, false, 2);
     else if (tiled) TILE_LAUNCH(float, false, 4);
     else
       paged_attention_kernel<float, false><<<grid, PA_RUN, 0, stream>>>(
-          (const float*)q, q_ld, Hq, Hkv, dh, (const float*)k_base, (const float*)v_base, page_stride, page_size,
-          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
+          (const float*)q, q_ld, Hq, Hkv, dh, dv, (const float*)k_base, (const float*)v_base, page_stride, page_size,
+          block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<float, false><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dh, runs, positions, window, (float*)out, out_ld);
+        partial, Hq, dv, runs, positions, window, sinks, (float*)out, out_ld);
   } else if (dtype == DT_BF16) {
     if (tiled && dims == 1) TILE_LAUNCH(bf16_t, true, 1);
     else if (tiled && dims == 2) TILE_LAUNCH(bf16_t, true, 2);
     else if (tiled) TILE_LAUNCH(bf16_t, true, 4);
     else
       paged_attention_kernel<bf16_t, true><<<grid, PA_RUN, 0, stream>>>(
-          (const bf16_t*)q, q_ld, Hq, Hkv, dh, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
-          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, runs, partial);
+          (const bf16_t*)q, q_ld, Hq, Hkv, dh, dv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride,
+          page_size, block_tables, max_pages, lane_of_token, positions, scale, window, slopes, log_bias, runs, partial);
     RETURN_IF_LAUNCH_FAILED();
     paged_attention_merge_kernel<bf16_t, true><<<merge_grid, merge_threads, 0, stream>>>(
-        partial, Hq, dh, runs, positions, window, (bf16_t*)out, out_ld);
+        partial, Hq, dv, runs, positions, window, sinks, (bf16_t*)out, out_ld);
   } else {
     return ERR_BAD_ARGUMENT;
   }

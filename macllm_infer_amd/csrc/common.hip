@@ -376,3 +376,129 @@ extern "C" int mi_add_bias_round(const float* sums, const float* bias, void* out
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
+
+// ---------------------------------------------------------------- scaled residual add + rmsnorm
+// add_rmsnorm for a branch that is multiplied, feature by feature, by a float32 vector where it joins the stream:
+//   v = h[r] + scale * delta[r] (the product and the sum in float32);  if no `rows`: h[r] = v;
+//   out[i] = v / sqrt(mean(v^2) + eps) * weight     (out may be null: the add alone).
+// One workgroup a row; a thread keeps its elements of the row in registers (up to SCALED_MAX_ROUNDS * 256 columns)
+// or, for wider rows, in LDS.  The sum of squares is added up in an order that d alone fixes.
+#define SCALED_MAX_ROUNDS 8
+template <typename TD, typename TO, bool IN_LDS>
+__global__ void __launch_bounds__(256)
+add_scaled_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ scale,
+                          const float* __restrict__ weight, float eps, TO* __restrict__ out,
+                          const int* __restrict__ rows, int d) {
+  extern __shared__ float wide_row[];
+  __shared__ float scratch[16];
+  const long out_row = blockIdx.x;
+  const long row = rows ? (long)rows[out_row] : out_row;
+  float* hr = h + row * d;
+  const TD* dr = delta + row * d;
+  float kept[SCALED_MAX_ROUNDS];
+  float sum_squares = 0.f;
+  if (IN_LDS) {
+    for (int i = threadIdx.x; i < d; i += 256) {
+      const float v = fmaf(scale[i], to_float(dr[i]), hr[i]);
+      if (!rows) hr[i] = v;
+      wide_row[i] = v;
+      sum_squares += v * v;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < SCALED_MAX_ROUNDS; ++r) {
+      const int i = (int)threadIdx.x + r * 256;
+      const int at = min(i, d - 1);
+      const float v = fmaf(scale[at], to_float(dr[at]), hr[at]);
+      kept[r] = v;
+      if (i < d) {
+        if (!rows) hr[i] = v;
+        sum_squares += v * v;
+      }
+    }
+  }
+  if (!out) return;
+  const float total = block_sum(sum_squares, scratch);
+  const float denominator = sqrtf(total / (float)d + eps);
+  TO* o = out + out_row * d;
+  if (IN_LDS) {
+    for (int i = threadIdx.x; i < d; i += 256) o[i] = from_float<TO>(wide_row[i] / denominator * weight[i]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < SCALED_MAX_ROUNDS; ++r) {
+      const int i = (int)threadIdx.x + r * 256;
+      if (i < d) o[i] = from_float<TO>(kept[r] / denominator * weight[i]);
+    }
+  }
+}
+
+extern "C" int mi_add_scaled_rmsnorm(float* h, const void* delta, int delta_dtype, const float* scale,
+                                     const float* weight, float eps, void* out, int out_dtype, const int* rows,
+                                     int n_rows, int d, hipStream_t stream) {
+  if (!h || !delta || !scale || !weight || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  const bool in_lds = d > 256 * SCALED_MAX_ROUNDS;
+  if (in_lds && (size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  const size_t lds = in_lds ? (size_t)d * sizeof(float) : 0;
+#define LAUNCH(TD, TO)                                                                                              \
+  do {                                                                                                              \
+    if (in_lds)                                                                                                     \
+      add_scaled_rmsnorm_kernel<TD, TO, true><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta, scale, weight, eps, \
+                                                                            (TO*)out, rows, d);                     \
+    else                                                                                                            \
+      add_scaled_rmsnorm_kernel<TD, TO, false><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta, scale, weight, eps,  \
+                                                                           (TO*)out, rows, d);                      \
+  } while (0)
+  if (delta_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
+  else if (delta_dtype == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == DT_BF16 && out_dtype == DT_F32) LAUNCH(bf16_t, float);
+  else return ERR_BAD_ARGUMENT;
+#undef LAUNCH
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- PolyNorm
+// out[t, i] = c0 * z / rms(z) + c1 * z^2 / rms(z^2) + c2 * z^3 / rms(z^3) + c3, with rms(x) = sqrt(mean over the
+// row of x^2 + eps): the three sums of squares of a token's row (z^2, z^4, z^6) in float32, one pass; the row is
+// read a second time (it is in cache) for the result.  One workgroup a row.
+template <typename T>
+__global__ void __launch_bounds__(256)
+polynorm_kernel(const T* __restrict__ z, long ld, const float* __restrict__ coefficients, float eps,
+                T* __restrict__ out, long out_ld, int I) {
+  __shared__ float scratch[16];
+  const T* zr = z + (long)blockIdx.x * ld;
+  float first = 0.f, second = 0.f, third = 0.f;
+  for (int i = threadIdx.x; i < I; i += 256) {
+    const float x = to_float(zr[i]);
+    const float x2 = x * x;
+    first += x2;
+    second += x2 * x2;
+    third += x2 * x2 * x2;
+  }
+  const float mean1 = block_sum(first, scratch) / (float)I;
+  const float mean2 = block_sum(second, scratch) / (float)I;
+  const float mean3 = block_sum(third, scratch) / (float)I;
+  const float a = coefficients[0] / sqrtf(mean1 + eps);
+  const float b = coefficients[1] / sqrtf(mean2 + eps);
+  const float c = coefficients[2] / sqrtf(mean3 + eps);
+  const float e = coefficients[3];
+  T* o = out + (long)blockIdx.x * out_ld;
+  for (int i = threadIdx.x; i < I; i += 256) {
+    const float x = to_float(zr[i]);
+    o[i] = from_float<T>(fmaf(x, fmaf(x, fmaf(x, c, b), a), e));
+  }
+}
+
+extern "C" int mi_polynorm(const void* z, int dtype, long ld, const float* coefficients, float eps, void* out,
+                           long out_ld, int T, int I, hipStream_t stream) {
+  if (!z || !coefficients || !out || T <= 0 || I <= 0 || ld < I || out_ld < I) return ERR_BAD_ARGUMENT;
+  if (dtype == DT_F32)
+    polynorm_kernel<float><<<T, 256, 0, stream>>>((const float*)z, ld, coefficients, eps, (float*)out, out_ld, I);
+  else if (dtype == DT_BF16)
+    polynorm_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)z, ld, coefficients, eps, (bf16_t*)out, out_ld, I);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

@@ -123,7 +123,10 @@ class Engine:
         if check_device:
             kernel_build.ensure_modules(DecoderModel.kernel_modules(self.spec) + list(kernel_build.HOST_MODULES))
         source.apply_aliases(self.spec.tensor_aliases, root_prefix=self.spec.root_namespace)
-        bound = bind(source, DecoderModel.expected_tensors(self.spec), DecoderModel.tensor_copies(self.spec))
+        expected = DecoderModel.expected_tensors(self.spec)
+        if self.spec.stored_name_rules:
+            source.apply_stored_names(self.spec.stored_name, [expect.name for expect in expected])
+        bound = bind(source, expected, DecoderModel.tensor_copies(self.spec))
         source.close()
         build = BuildContext(hidden_size=self.spec.hidden_size, dtype=self.dtype, device=self.device,
                              max_context=self.spec.max_context, measure_paths=measured_paths)

@@ -12,6 +12,7 @@ from dataclasses import dataclass
 ATTENTION_MAX_HEAD_DIM = 256      # ATT_MAX_DH in attention.hip: a query row in LDS, head_dim / 64 sums a lane
 CONV_MAX_TAPS = 16                # CONV_MAX_K in mamba2.hip: the taps of a channel in registers
 SCAN_MAX_STATE = 512              # WAVE * SCAN_MAX_PER_THREAD in mamba2.hip: a state row over one wave
+LINEAR_STATE_MAX_KEY_DIM = 1024   # LS_MAX_PER_LANE * WAVE in linear_state.hip: a state column over one wave
 NORM_MAX_WIDTH = 16384            # 64 KiB of LDS hold a float32 row in common.hip's norm
 GRID_MOST = 65535                 # heads, groups or lanes that index a launch's y or z dimension
 

@@ -40,13 +40,24 @@ _SIGNATURES = {
         "mi_scale_to_f32": [_c_ptr, _c_int, _c_float, _c_ptr, _c_long, _c_ptr],
         "mi_tanh_softcap": [_c_ptr, _c_float, _c_long, _c_ptr],
         "mi_add_bias_round": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_add_scaled_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
+                                  _c_ptr],
+        "mi_polynorm": [_c_ptr, _c_int, _c_long, _c_ptr, _c_float, _c_ptr, _c_long, _c_int, _c_int, _c_ptr],
+    },
+    "linear_state": {
+        "mi_linear_state_scan": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                                 _c_ptr, _c_ptr, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int,
+                                 _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_ptr],
+        "mi_head_norm_gate": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr,
+                              _c_long, _c_int, _c_ptr],
+        "mi_tanh_rows": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_int, _c_int, _c_ptr],
     },
     "attention": {
-        "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
+        "mi_rope_kv_store": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int,
                              _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr],
-        "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
-                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_int, _c_ptr, _c_long,
-                               _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
+        "mi_paged_attention": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long,
+                               _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                               _c_ptr, _c_long, _c_ptr, _c_long, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr],
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
@@ -284,6 +295,124 @@ def tanh_softcap(logits: torch.Tensor, cap: float) -> None:
         _check(_fn("common", "mi_tanh_softcap")(_p(logits), float(cap), logits.numel(), _stream()), "tanh_softcap")
 
 
+def add_scaled_rmsnorm(h: torch.Tensor, delta: torch.Tensor, scale: torch.Tensor, weight: torch.Tensor, eps: float,
+                       out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+    """h += scale * delta (float32, in place; ``scale`` float32 [d], one factor a feature);
+    out = h / sqrt(mean(h^2) + eps) * weight.  With ``rows`` only those rows are read, ``out[i]`` gets row
+    ``rows[i]`` and ``h`` is left as it is.  ``out`` may be None when only the sum is wanted."""
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and h.is_cuda,
+          "add_scaled_rmsnorm: h must be contiguous float32 [T, d]")
+    T, d = h.shape
+    _need(delta.shape == h.shape and delta.is_contiguous(), "add_scaled_rmsnorm: delta must be contiguous [T, d]")
+    for name, vector in (("scale", scale), ("weight", weight)):
+        _need(vector.dtype == torch.float32 and vector.numel() == d and vector.is_contiguous() and vector.is_cuda,
+              f"add_scaled_rmsnorm: {name} must be float32 [d] on the GPU")
+    n_rows = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+        _need(out is not None, "add_scaled_rmsnorm: a gather needs somewhere to put its rows")
+    if out is not None:
+        _need(out.shape == (n_rows, d) and out.is_contiguous(), "add_scaled_rmsnorm: out must be contiguous [rows, d]")
+    _check(_fn("common", "mi_add_scaled_rmsnorm")(
+        _p(h), _p(delta), _dt(delta), _p(scale), _p(weight), float(eps), _p(out),
+        _dt(out) if out is not None else DT_F32, _p(rows), n_rows, d, _stream()), "add_scaled_rmsnorm", f"(d={d})")
+
+
+def polynorm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = c0 z/rms(z) + c1 z^2/rms(z^2) + c2 z^3/rms(z^3) + c3 row by row, rms(x) = sqrt(mean(x^2) + eps)
+    over the row; ``coefficients`` float32 [4]."""
+    ld = _row_major(z, "z")
+    out_ld = _row_major(out, "out")
+    _need(out.shape == z.shape and out.dtype == z.dtype, "polynorm: out must have the input's shape and dtype")
+    _need(coefficients.dtype == torch.float32 and coefficients.numel() == 4 and coefficients.is_cuda
+          and coefficients.is_contiguous(), "polynorm: coefficients must be float32 [4] on the GPU")
+    _check(_fn("common", "mi_polynorm")(_p(z), _dt(z), ld, _p(coefficients), float(eps), _p(out), out_ld, z.shape[0],
+                                        z.shape[1], _stream()), "polynorm")
+
+
+# --------------------------------------------------------------------------- mixers with a matrix-valued state
+def tanh_rows(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = tanh(x) for a block of columns (``x`` may be a column view of a wider matrix)."""
+    ld = _row_major(x, "x")
+    out_ld = _row_major(out, "out")
+    _need(out.shape == x.shape and out.dtype == x.dtype, "tanh_rows: out must have the input's shape and dtype")
+    _check(_fn("linear_state", "mi_tanh_rows")(_p(x), _dt(x), ld, _p(out), out_ld, x.shape[0], x.shape[1], _stream()),
+           "tanh_rows")
+
+
+def head_norm_gate(raw: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], num_heads: int, eps: float,
+                   activation: str, out: torch.Tensor) -> None:
+    """out[t, head] = raw[t, head] / rms(raw[t, head]) (* weight) * act(gate[t, head]) with rms over the head's
+    columns and act "silu" or "sigmoid".  ``raw`` float32 [T, H * dv]; ``gate`` and ``out`` [T, H * dv] of the
+    activation dtype (column views allowed); ``weight`` float32 [H * dv] or None."""
+    raw_ld = _row_major(raw, "raw")
+    gate_ld = _row_major(gate, "gate")
+    out_ld = _row_major(out, "out")
+    T, width = raw.shape
+    _need(raw.dtype == torch.float32 and width % num_heads == 0 and gate.shape == raw.shape and out.shape == raw.shape
+          and gate.dtype == out.dtype, "head_norm_gate: shapes or dtypes do not match")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.numel() == width and weight.is_contiguous()
+                             and weight.is_cuda), "head_norm_gate: weight must be float32 [H * dv] on the GPU")
+    _need(activation in ("silu", "sigmoid"), "head_norm_gate: the gate's activation is 'silu' or 'sigmoid'")
+    _check(_fn("linear_state", "mi_head_norm_gate")(
+        _p(raw), raw_ld, _p(gate), _dt(gate), gate_ld, _p(weight), num_heads, width // num_heads, float(eps),
+        0 if activation == "silu" else 1, _p(out), out_ld, T, _stream()), "head_norm_gate")
+
+
+def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, num_heads: int, key_dim: int,
+                      value_dim: int, state: torch.Tensor, cu_seqlens: torch.Tensor, slot_ids: torch.Tensor,
+                      out: torch.Tensor, max_query_len: int = 0, head_decay: Optional[torch.Tensor] = None,
+                      key_scale: float = 1.0, positions: Optional[torch.Tensor] = None,
+                      inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0, removal_col: int = -1,
+                      decay_logits: Optional[torch.Tensor] = None, decay_bias: Optional[torch.Tensor] = None,
+                      decay_floor: float = 0.0, key_eps: float = 0.0) -> None:
+    """The scan of a mixer whose state is a matrix per head, from and into ``state`` [slots, H, dv, dk] (float32, the
+    state of a head transposed), for every lane of the step from its slot; ``out`` float32 [T, H * dv] = S^T q.
+
+    ``u`` [T, ...]: the projection's rows with q heads at ``q_col``, k heads at ``k_col`` (H * dk columns each) and
+    v heads at ``v_col`` (H * dv).  Retention (``head_decay`` float32 [H]): S <- decay S + k v^T after q and k were
+    turned by ``positions`` (``inv_freq``, ``rotary_dim``; None: no rotation) and k multiplied by ``key_scale``.
+    Delta rule (``removal_col`` >= 0: the columns of the removal rate's logits; ``decay_logits`` float32 [T, H * dk],
+    ``decay_bias`` float32 [H * dk]): w = exp(-decay_floor * sigmoid(logits + bias)), a = sigmoid(removal),
+    u = k / sqrt(sum k^2 + key_eps), S <- diag(w) S - (a u)(u^T S) + k v^T.  ``max_query_len``: the longest lane
+    (1 picks small workgroups; 0: not known)."""
+    ld = _row_major(u, "u")
+    T = u.shape[0]
+    H, dk, dv = int(num_heads), int(key_dim), int(value_dim)
+    delta = removal_col >= 0
+    widest = max(q_col + H * dk, k_col + H * dk, v_col + H * dv, removal_col + H * dk if delta else 0)
+    _need(min(q_col, k_col, v_col) >= 0 and u.shape[1] >= widest, "linear_state_scan: u is too narrow for its columns")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.shape[1:] == (H, dv, dk) and state.is_contiguous()
+          and state.is_cuda, "linear_state_scan: state must be contiguous float32 [slots, H, dv, dk] on the GPU")
+    _i32(cu_seqlens, "cu_seqlens")
+    _i32(slot_ids, "slot_ids")
+    lanes = slot_ids.numel()
+    _need(cu_seqlens.numel() == lanes + 1, "linear_state_scan: one offset more than lanes")
+    _need(out.dtype == torch.float32 and out.shape == (T, H * dv) and out.is_contiguous(),
+          "linear_state_scan: out must be contiguous float32 [T, H * dv]")
+    logits_ld = 0
+    if delta:
+        _need(decay_logits is not None and decay_logits.dtype == torch.float32 and decay_logits.shape == (T, H * dk),
+              "linear_state_scan: decay_logits must be float32 [T, H * dk]")
+        logits_ld = _row_major(decay_logits, "decay_logits")
+        _need(decay_bias is not None and decay_bias.dtype == torch.float32 and decay_bias.numel() == H * dk
+              and decay_bias.is_contiguous() and decay_bias.is_cuda, "linear_state_scan: decay_bias must be float32 [H * dk]")
+    else:
+        _need(head_decay is not None and head_decay.dtype == torch.float32 and head_decay.numel() == H
+              and head_decay.is_cuda, "linear_state_scan: head_decay must be float32 [H] on the GPU")
+    if inv_freq is not None:
+        _i32(positions, "positions")
+        _need(positions.numel() == T and inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2
+              and inv_freq.is_cuda and 0 < rotary_dim <= dk, "linear_state_scan: the rotation does not fit the heads")
+    _check(_fn("linear_state", "mi_linear_state_scan")(
+        _p(u), _dt(u), ld, int(q_col), int(k_col), int(v_col), int(removal_col), H, dk, dv, _p(state), _p(cu_seqlens),
+        _p(slot_ids), lanes, _p(out), out.stride(0), int(max_query_len), _p(head_decay), float(key_scale),
+        _p(positions) if inv_freq is not None else None, _p(inv_freq), int(rotary_dim) if inv_freq is not None else 0,
+        _p(decay_logits), logits_ld, _p(decay_bias), float(decay_floor), float(key_eps), _stream()),
+        "linear_state_scan", f"(dk={dk}, dv={dv})")
+
+
 # --------------------------------------------------------------------------- matrix products
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], keep_float32: bool = False) -> torch.Tensor:
     """x [M, K] . weight[N, K]^T (+ bias float32 [N]) -> [M, N] in x's dtype, or, with
@@ -326,15 +455,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
 def rope_kv_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                   positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rotary_dim: int,
                   slot_mapping: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
-                  v_cache: Optional[torch.Tensor]) -> None:
+                  v_cache: Optional[torch.Tensor], value_dim: Optional[int] = None) -> None:
     """Rotate q (in place) and k of every token; store rotated k and raw v into the cache.
 
-    ``qkv`` [T, >= (Hq+2Hkv)*dh] holds q heads, k heads, v heads.  ``k_cache`` [pages, Hkv,
-    page_size, dh] and ``v_cache`` [pages, Hkv, dh, page_size] are one layer's views of the pool;
+    ``qkv`` [T, >= (Hq+Hkv)*dh + Hkv*dv] holds q heads, k heads, v heads (``value_dim`` dv: the width of a value
+    head, the keys' if not given).  ``k_cache`` [pages, Hkv,
+    page_size, dh] and ``v_cache`` [pages, Hkv, dv, page_size] are one layer's views of the pool;
     ``slot_mapping[t] = page*page_size + offset``.  Without ``slot_mapping`` nothing is stored."""
     ld = _row_major(qkv, "qkv")
     T = qkv.shape[0]
-    _need(qkv.shape[1] >= (num_heads + 2 * num_kv_heads) * head_dim, "rope_kv_store: qkv is too narrow")
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    _need(qkv.shape[1] >= (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim,
+          "rope_kv_store: qkv is too narrow")
     _i32(positions, "positions")
     _need(positions.numel() == T, "rope_kv_store: one position per token")
     if inv_freq is not None:
@@ -344,26 +476,28 @@ def rope_kv_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     if slot_mapping is not None:
         _i32(slot_mapping, "slot_mapping")
         _need(slot_mapping.numel() == T, "rope_kv_store: one cache cell per token")
-        page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype)
+        page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype, value_dim)
     _check(_fn("attention", "mi_rope_kv_store")(
-        _p(qkv), _dt(qkv), ld, T, num_heads, num_kv_heads, head_dim, _p(positions), _p(inv_freq),
+        _p(qkv), _dt(qkv), ld, T, num_heads, num_kv_heads, head_dim, value_dim, _p(positions), _p(inv_freq),
         rotary_dim if inv_freq is not None else 0, _p(slot_mapping),
         _p(k_cache) if slot_mapping is not None else None, _p(v_cache) if slot_mapping is not None else None,
         page_stride, page_size, _stream()), "rope_kv_store")
 
 
-def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype):
-    """K pages are [pages, Hkv, page_size, dh]; V pages are transposed, [pages, Hkv, dh, page_size]."""
+def _cache_view(k_cache, v_cache, num_kv_heads, head_dim, dtype, value_dim=None):
+    """K pages are [pages, Hkv, page_size, dh]; V pages are transposed, [pages, Hkv, dv, page_size] (dv the
+    width of a value head: ``value_dim``, or the keys')."""
+    value_dim = head_dim if value_dim is None else value_dim
     _need(k_cache is not None and v_cache is not None and k_cache.dim() == 4 and v_cache.dim() == 4,
-          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dh, page_size]")
+          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dv, page_size]")
     page_size = k_cache.shape[2]
     _need(k_cache.shape[1] == num_kv_heads and k_cache.shape[3] == head_dim
-          and v_cache.shape == (k_cache.shape[0], num_kv_heads, head_dim, page_size),
-          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dh, page_size]")
-    for name, cache in (("k_cache", k_cache), ("v_cache", v_cache)):
+          and v_cache.shape == (k_cache.shape[0], num_kv_heads, value_dim, page_size),
+          "k_cache must be [pages, Hkv, page_size, dh] and v_cache [pages, Hkv, dv, page_size]")
+    for name, cache, width in (("k_cache", k_cache, head_dim), ("v_cache", v_cache, value_dim)):
         _need(cache.dtype == dtype and cache.is_cuda, f"{name} must be a GPU tensor of the activation dtype")
         _need(cache.stride(3) == 1 and cache.stride(2) == cache.shape[3]
-              and cache.stride(1) == page_size * head_dim, f"{name}: a page's block per kv head must be dense")
+              and cache.stride(1) == page_size * width, f"{name}: a page's block per kv head must be dense")
     _need(k_cache.stride(0) == v_cache.stride(0), "k_cache and v_cache must share a page stride")
     return k_cache.stride(0), page_size
 
@@ -373,7 +507,9 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
                     lane_of_token: torch.Tensor, positions: torch.Tensor, scale: float,
                     window: Optional[int], out: torch.Tensor, max_seq_len: Optional[int] = None,
                     slopes: Optional[torch.Tensor] = None, query_tiles: Optional[torch.Tensor] = None,
-                    tile_tokens: int = 0, cu_seqlens: Optional[torch.Tensor] = None) -> None:
+                    tile_tokens: int = 0, cu_seqlens: Optional[torch.Tensor] = None,
+                    log_bias: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
+                    value_dim: Optional[int] = None) -> None:
     """Causal attention of every token over its request's cached keys (its own included).
 
     ``q`` [T, >= Hq*dh] (rotated); ``block_tables`` [lanes, max_pages] page ids by logical
@@ -383,13 +519,17 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
     the work area, never the result.  ``slopes`` (float32 [Hq]): a bias on the scores by distance,
     ``score -= slopes[head] * (s - p)``.  ``query_tiles`` [tiles, 2] = (lane or -1, first token row) of runs of
     up to ``tile_tokens`` tokens of one lane, with ``cu_seqlens`` [lanes + 1]: for steps whose lanes hold several
-    tokens, a kernel that fetches a run of keys once for sixteen queries (the same bits as without)."""
+    tokens, a kernel that fetches a run of keys once for sixteen queries (the same bits as without).
+    ``log_bias`` (float32 [Hq, 2] = (r1, r2)): ``score -= r1 * ln(1 + r2 * (s - p))``.  ``sinks`` (float32 [Hq]):
+    exp(sink) is one more term of the softmax's denominator, with no key and no value.  ``value_dim``: the
+    width of a value head if it is not the keys'; ``out`` is then [T, Hq * value_dim]."""
     q_ld = _row_major(q, "q")
     out_ld = _row_major(out, "out")
     T = q.shape[0]
-    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * head_dim)
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    _need(q.shape[1] >= num_heads * head_dim and out.shape == (T, num_heads * value_dim)
           and out.dtype == q.dtype, "paged_attention: q/out shapes do not match")
-    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+    page_stride, page_size = _cache_view(k_cache, v_cache, num_kv_heads, head_dim, q.dtype, value_dim)
     _i32(block_tables, "block_tables")
     _i32(lane_of_token, "lane_of_token")
     _i32(positions, "positions")
@@ -397,9 +537,14 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
           "paged_attention: metadata shapes do not match")
     _need(slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == num_heads and slopes.is_contiguous()
                              and slopes.is_cuda), "paged_attention: slopes must be float32 [Hq] on the GPU")
+    _need(log_bias is None or (log_bias.dtype == torch.float32 and log_bias.shape == (num_heads, 2)
+                               and log_bias.is_contiguous() and log_bias.is_cuda),
+          "paged_attention: log_bias must be float32 [Hq, 2] on the GPU")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads and sinks.is_contiguous()
+                            and sinks.is_cuda), "paged_attention: sinks must be float32 [Hq] on the GPU")
     holds = block_tables.shape[1] * page_size
     span = holds if max_seq_len is None else max(1, min(int(max_seq_len), holds))
-    floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, head_dim, span)
+    floats = _fn("attention", "mi_paged_attention_workspace", _c_long)(T, num_heads, value_dim, span)
     partial = torch.empty((max(int(floats), 1),), dtype=torch.float32, device=q.device)
     tiles = 0
     if query_tiles is not None and tile_tokens and tile_tokens % 16 == 0 and cu_seqlens is not None:
@@ -409,9 +554,9 @@ def paged_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim
               "paged_attention: the table of runs or the lanes' offsets do not fit the step")
         tiles = query_tiles.shape[0]
     _check(_fn("attention", "mi_paged_attention")(
-        _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride,
+        _p(q), _dt(q), q_ld, T, num_heads, num_kv_heads, head_dim, value_dim, _p(k_cache), _p(v_cache), page_stride,
         page_size, _p(block_tables), block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale),
-        int(window or 0), _p(slopes), span, _p(partial), partial.numel(), _p(out), out_ld,
+        int(window or 0), _p(slopes), _p(log_bias), _p(sinks), span, _p(partial), partial.numel(), _p(out), out_ld,
         _p(query_tiles) if tiles else None, tiles, int(tile_tokens) if tiles else 0, _p(cu_seqlens) if tiles else None,
         _stream()), "paged_attention", f"(head_dim={head_dim})")
 

@@ -19,6 +19,10 @@ class Attention(Mixer):
     (reference: src/decoder.rs:1099-1161 projections, :953-962 RoPE and cache write,
     :4580-4670 scores with float32 softmax, :923-931 output; GQA pairing :4641-4647.)
 
+    Values may have a width of their own (``value_dim``), the softmax may hold a sink (``sink``: a learned number
+    per query head whose exponential is one more term of the denominator, with no key and no value), and the
+    position encoding may be a bias on the scores; all three take the general attention kernel.
+
     Multipliers: ``in_multiplier`` scales the input of q/k/v (folded into their weights),
     ``key_multiplier`` the k projection's output (weights and bias), ``out_multiplier``
     the output projection's output."""
@@ -30,54 +34,70 @@ class Attention(Mixer):
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
         q_rows = spec.num_heads * spec.head_dim
         kv_rows = spec.num_kv_heads * spec.head_dim
+        v_rows = spec.num_kv_heads * spec.value_width
         out = [Expect(f"{prefix}.q_proj.weight", ((q_rows, hidden_size),)),
                Expect(f"{prefix}.k_proj.weight", ((kv_rows, hidden_size),)),
-               Expect(f"{prefix}.v_proj.weight", ((kv_rows, hidden_size),)),
-               Expect(f"{prefix}.o_proj.weight", ((hidden_size, q_rows),))]
+               Expect(f"{prefix}.v_proj.weight", ((v_rows, hidden_size),)),
+               Expect(f"{prefix}.o_proj.weight", ((hidden_size, spec.num_heads * spec.value_width),))]
         if spec.qkv_bias:
             out += [Expect(f"{prefix}.q_proj.bias", ((q_rows,),), init="bias"),
                     Expect(f"{prefix}.k_proj.bias", ((kv_rows,),), init="bias"),
-                    Expect(f"{prefix}.v_proj.bias", ((kv_rows,),), init="bias")]
+                    Expect(f"{prefix}.v_proj.bias", ((v_rows,),), init="bias")]
         if spec.out_bias:
             out.append(Expect(f"{prefix}.o_proj.bias", ((hidden_size,),), init="bias"))
+        if spec.sink:
+            out.append(Expect(f"{prefix}.sink", ((spec.num_heads,),), init="logit"))
+        out += part_class(spec.position).expected_tensors(spec.position, prefix, hidden_size)
         return out
 
     @classmethod
     def limits(cls, spec, hidden_size: int):
-        return (beyond("attention", "head_dim", spec.head_dim, ATTENTION_MAX_HEAD_DIM,
+        return (beyond("attention", "head_dim", max(spec.head_dim, spec.value_width), ATTENTION_MAX_HEAD_DIM,
                        "a query row and its sums are kept in LDS and registers")
                 + beyond("attention", "num_heads", spec.num_heads, GRID_MOST, "heads index a dimension of the launch")
                 + part_class(spec.position).limits(spec.position, spec.head_dim))
 
     @classmethod
     def cache_needs(cls, spec):
-        return [KVNeed(spec.num_kv_heads, spec.head_dim, spec.window)]
+        return [KVNeed(spec.num_kv_heads, spec.head_dim, spec.window,
+                       None if spec.value_width == spec.head_dim else spec.value_width)]
 
     def __init__(self, spec, prefix: str, tensors, build: BuildContext):
         self.spec = spec
         self.build = build
         q_rows = spec.num_heads * spec.head_dim
         kv_rows = spec.num_kv_heads * spec.head_dim
+        v_rows = spec.num_kv_heads * spec.value_width
         get = lambda name: tensors.get(f"{prefix}.{name}")
         weight_scale = torch.cat([torch.full((q_rows,), spec.in_multiplier),
                                   torch.full((kv_rows,), spec.in_multiplier * spec.key_multiplier),
-                                  torch.full((kv_rows,), spec.in_multiplier)])
+                                  torch.full((v_rows,), spec.in_multiplier)])
         bias_scale = torch.cat([torch.ones(q_rows), torch.full((kv_rows,), spec.key_multiplier),
-                                torch.ones(kv_rows)])
+                                torch.ones(v_rows)])
         self.qkv = Linear([get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")],
                           [get("q_proj.bias"), get("k_proj.bias"), get("v_proj.bias")], build,
                           weight_scale=weight_scale, bias_scale=bias_scale)
         self.out = Linear([get("o_proj.weight")], [get("o_proj.bias")], build,
                           weight_scale=spec.out_multiplier, bias_scale=spec.out_multiplier)
-        self.position = part_class(spec.position)(spec.position, spec.head_dim, build)
+        position_class = part_class(spec.position)
+        if getattr(position_class, "learned", False):        # an encoding with tensors of its own, beside the mixer's
+            self.position = position_class(spec.position, spec.head_dim, build, prefix=prefix, tensors=tensors)
+        else:
+            self.position = position_class(spec.position, spec.head_dim, build)
+        self.sink = get("sink").to(torch.float32).contiguous().to(build.device) if spec.sink else None
         self.graph_safe = bool(getattr(self.position, "graph_safe", False))
+        # what only the general kernel knows: a bias on the scores, a sink, values of another width than the keys
+        self.general_only = (self.position.score_slopes is not None or self.position.score_log_bias is not None
+                             or self.sink is not None or spec.value_width != spec.head_dim)
 
     def projections(self):
+        if self.general_only:          # the fused decode kernels know none of it: the layer runs part by part
+            return None
         return self.qkv, self.out, self.spec.num_heads * self.spec.head_dim
 
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         spec = self.spec
-        attended = torch.empty((x.shape[0], spec.num_heads * spec.head_dim), dtype=x.dtype, device=x.device)
+        attended = torch.empty((x.shape[0], spec.num_heads * spec.value_width), dtype=x.dtype, device=x.device)
         self.mix(self.qkv(x), step, cache, attended)
         return self.out(attended)
 
@@ -85,9 +105,22 @@ class Attention(Mixer):
         """From the projected rows [q | k | v] (rotated and stored in place) to the attended rows
         ``attended`` [T, Hq * dh]; both may be column views of wider matrices."""
         spec = self.spec
-        self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
         geometry = (spec.num_heads, spec.num_kv_heads, spec.head_dim)
         slopes = self.position.score_slopes
+        if self.general_only:
+            self.position.rotate(qkv, *geometry, step)
+            if cache.owns_kv:
+                ops.rope_kv_store(qkv, *geometry, step.positions, None, 0, step.slot_mappings[cache.group],
+                                  cache.k_cache, cache.v_cache, value_dim=spec.value_width)
+            tiles = {}
+            if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
+                tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
+            ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                step.lane_of_token, step.positions, spec.scale, spec.window, attended,
+                                step.max_seq_len, slopes, log_bias=self.position.score_log_bias, sinks=self.sink,
+                                value_dim=spec.value_width, **tiles)
+            return
+        self.position.rotate_and_store(qkv, spec.num_heads, spec.num_kv_heads, spec.head_dim, step, cache)
         # lanes of several tokens: the general kernel shares a run of keys among the queries of a tile of the step's
         # table of runs (when the step was packed with one)
         tiles = {}

@@ -72,9 +72,17 @@ class ScaledRows:
     weight: torch.Tensor
 
 
+@dataclass
+class ScaledBranch:
+    """A branch output [T, d] that is multiplied, feature by feature, by ``scale`` (float32 [d]) where it is added
+    to the residual stream: an entry of ``Residual.pending`` in place of the plain tensor."""
+    rows: torch.Tensor
+    scale: torch.Tensor
+
+
 class Residual:
-    """The float32 residual stream [T, d] plus the branch outputs not yet added to it.
-    The next norm adds them and normalizes in one kernel.
+    """The float32 residual stream [T, d] plus the branch outputs not yet added to it (tensors, or
+    ``ScaledBranch``es).  The next norm adds them and normalizes in one kernel.
 
     ``next_norm``: (weight, eps) of the norm that the layer after the one running starts with (the final norm
     after the last), if that norm is a root-mean-square norm, set by whoever runs the layers; a layer whose last

@@ -5,7 +5,8 @@ from typing import Dict
 
 import torch
 
-from .base import BuildContext, Residual, part_class
+from ..weights.loader import Expect
+from .base import BuildContext, Residual, ScaledBranch, part_class
 
 _ARRANGEMENTS: Dict[str, type] = {}
 _FUSIONS: Dict[str, object] = {}
@@ -66,7 +67,9 @@ class ParallelPreNormBlock:
     """n = norm(h); h += sum over mixers of mixer(n); h += ffn(norm(h)).
     All mixers read the same normed input and their outputs are summed into the residual
     (reference: src/decoder.rs:2658-2682, 2684-2699).  With one mixer this is the ordinary
-    sequential pre-norm layer."""
+    sequential pre-norm layer.  A layer may scale either branch feature by feature before the add
+    (``mixer_scale_name`` / ``ffn_scale_name``: h += scale * branch, the product in float32), and may have no
+    feed-forward at all (``ffn`` None)."""
 
     @classmethod
     def expected_tensors(cls, layer, hidden_size: int):
@@ -75,23 +78,36 @@ class ParallelPreNormBlock:
             layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}", hidden_size)
         for slot in layer.mixers:
             out += part_class(slot.spec).expected_tensors(slot.spec, f"{layer.prefix}.{slot.name}", hidden_size)
-        out += part_class(layer.ffn_norm).expected_tensors(
+        if layer.mixer_scale_name:
+            out.append(Expect(f"{layer.prefix}.{layer.mixer_scale_name}", ((hidden_size,),), init="scale"))
+        second = part_class(layer.ffn_norm).expected_tensors(
             layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", hidden_size)
+        if layer.ffn_scale_name:
+            second.append(Expect(f"{layer.prefix}.{layer.ffn_scale_name}", ((hidden_size,),), init="scale"))
+        if layer.ffn is None:
+            # a layer without a feed-forward uses neither; a checkpoint that holds them all the same is accepted
+            return out + [Expect(one.name, one.shapes, one.init, one.integer, optional=True) for one in second]
+        out += second
         out += part_class(layer.ffn).expected_tensors(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", hidden_size)
         return out
+
+    @staticmethod
+    def _part_specs(layer):
+        second = [] if layer.ffn is None else [layer.ffn_norm, layer.ffn]
+        return [layer.mixer_norm] + second + [slot.spec for slot in layer.mixers]
 
     @classmethod
     def limits(cls, layer, hidden_size: int):
         """What the kernels of this layer's parts refuse (see ``Part.limits``)."""
         out = []
-        for spec in [layer.mixer_norm, layer.ffn_norm, layer.ffn] + [slot.spec for slot in layer.mixers]:
+        for spec in cls._part_specs(layer):
             out += part_class(spec).limits(spec, hidden_size)
         return out
 
     @classmethod
     def kernel_modules(cls, layer):
         modules = []
-        for spec in [layer.mixer_norm, layer.ffn_norm, layer.ffn] + [slot.spec for slot in layer.mixers]:
+        for spec in cls._part_specs(layer):
             modules += list(part_class(spec).kernel_modules)
         return modules
 
@@ -101,15 +117,27 @@ class ParallelPreNormBlock:
             layer.mixer_norm, f"{layer.prefix}.{layer.mixer_norm_name}", tensors, build)
         self.mixers = [(slot.name, part_class(slot.spec)(slot.spec, f"{layer.prefix}.{slot.name}", tensors, build))
                        for slot in layer.mixers]
-        self.ffn_norm = part_class(layer.ffn_norm)(
-            layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
-        self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
+        self.ffn_norm = self.ffn = None
+        if layer.ffn is not None:
+            self.ffn_norm = part_class(layer.ffn_norm)(
+                layer.ffn_norm, f"{layer.prefix}.{layer.ffn_norm_name}", tensors, build)
+            self.ffn = part_class(layer.ffn)(layer.ffn, f"{layer.prefix}.{layer.ffn_name}", tensors, build)
+
+        def scale(name):
+            if not name:
+                return None
+            return tensors[f"{layer.prefix}.{name}"].to(torch.float32).contiguous().to(build.device)
+        self.mixer_scale = scale(layer.mixer_scale_name)
+        self.ffn_scale = scale(layer.ffn_scale_name) if layer.ffn is not None else None
         factory = _FUSIONS.get(layer.arrangement)
-        self.fusion = factory(self, build) if factory is not None else None      # None when parts or sizes do not fit
+        # the fast path knows plain branches and a feed-forward behind them; None when parts or sizes do not fit
+        plain = self.mixer_scale is None and self.ffn_scale is None and self.ffn is not None
+        self.fusion = factory(self, build) if factory is not None and plain else None
 
     @property
     def graph_safe(self) -> bool:
-        parts = [self.mixer_norm, self.ffn_norm, self.ffn] + [mixer for _, mixer in self.mixers]
+        parts = [self.mixer_norm] + [mixer for _, mixer in self.mixers]
+        parts += [self.ffn_norm, self.ffn] if self.ffn is not None else []
         return all(getattr(part, "graph_safe", False) for part in parts)
 
     def tune(self, peers) -> None:
@@ -141,8 +169,14 @@ class ParallelPreNormBlock:
             with torch.cuda.stream(side):
                 first_out = first.forward(normed, step, caches[first_name])
             main.wait_stream(side)
-            residual.pending = [first_out, second_out]
+            outputs = [first_out, second_out]
         else:
-            residual.pending = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+            outputs = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
+        if self.mixer_scale is not None:
+            outputs = [ScaledBranch(rows, self.mixer_scale) for rows in outputs]
+        residual.pending = outputs
+        if self.ffn is None:
+            return
         normed = self.ffn_norm.forward(residual)
-        residual.pending = [self.ffn.forward(normed)]
+        rows = self.ffn.forward(normed)
+        residual.pending = [rows if self.ffn_scale is None else ScaledBranch(rows, self.ffn_scale)]

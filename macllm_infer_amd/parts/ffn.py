@@ -56,3 +56,31 @@ class SwiGLU(FeedForward):
         activated = torch.empty((x.shape[0], self.spec.intermediate_size), dtype=gate_up.dtype, device=x.device)
         ops.swiglu(gate_up, activated, self.tile)
         return self.down(activated)
+
+
+@register_part("polynorm_ffn")
+class PolyNormFFN(FeedForward):
+    """down(act(up(x))) with act(z) = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3: powers element by element, N divides
+    a token's row of inner values by its root mean square (three sums of squares over the row, in float32, one
+    kernel).  The four numbers are the tensor ``act``."""
+    graph_safe = True
+    kernel_modules = ("common", "gemm")
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        inner = spec.intermediate_size
+        return [Expect(f"{prefix}.up.weight", ((inner, hidden_size),)),
+                Expect(f"{prefix}.down.weight", ((hidden_size, inner),)),
+                Expect(f"{prefix}.act", ((4,),), init="scale")]
+
+    def __init__(self, spec, prefix: str, tensors, build: BuildContext):
+        self.spec = spec
+        self.up = Linear([tensors[f"{prefix}.up.weight"]], [None], build)
+        self.down = Linear([tensors[f"{prefix}.down.weight"]], [None], build)
+        self.coefficients = tensors[f"{prefix}.act"].to(torch.float32).contiguous().to(build.device)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        inner = self.up(x)
+        activated = torch.empty_like(inner)
+        ops.polynorm(inner, self.coefficients, self.spec.eps, activated)
+        return self.down(activated)

@@ -8,13 +8,13 @@ import torch
 from ..kernels import ops
 from ..kernels.limits import NORM_MAX_WIDTH, beyond
 from ..weights.loader import Expect
-from .base import BuildContext, Part, Residual, register_part
+from .base import BuildContext, Part, Residual, ScaledBranch, register_part
 
 
 def partial_slab(pending) -> Optional[torch.Tensor]:
     """The float32 [S, T, d] tensor whose slabs, in order, ``pending`` lists (a branch that arrives as
     partial sums of a product split over K), or None."""
-    if len(pending) < 2:
+    if len(pending) < 2 or any(isinstance(branch, ScaledBranch) for branch in pending):
         return None
     base = pending[0]._base
     if (base is None or base.dim() != 3 or base.dtype != torch.float32 or base.shape[0] != len(pending)
@@ -28,14 +28,15 @@ def partial_slab(pending) -> Optional[torch.Tensor]:
 
 @register_part("rmsnorm")
 class RmsNorm(Part):
-    """y = x / sqrt(mean(x^2) + eps) * w, statistics in float32
-    (reference: src/model_weights.rs:563-565, golden src/decoder.rs:10331-10334)."""
+    """y = x / sqrt(mean(x^2) + eps) * (w + weight_offset), statistics in float32
+    (reference: src/model_weights.rs:563-565, golden src/decoder.rs:10331-10334).  The offset (1 for a weight
+    stored around zero) is added once, in float32, when the part is built."""
     graph_safe = True
     kernel_modules = ("common",)
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
-        return [Expect(f"{prefix}.weight", ((hidden_size,),), init="norm")]
+        return [Expect(f"{prefix}.weight", ((hidden_size,),), init="zero_centred" if spec.weight_offset else "norm")]
 
     @classmethod
     def limits(cls, spec, hidden_size: int):
@@ -44,7 +45,13 @@ class RmsNorm(Part):
     def __init__(self, spec, prefix: str, tensors, build: BuildContext):
         self.eps = spec.eps
         self.build = build
-        self.weight = tensors[f"{prefix}.weight"].to(torch.float32).contiguous().to(build.device)
+        self.weight = (tensors[f"{prefix}.weight"].to(torch.float32) + float(spec.weight_offset)).contiguous().to(build.device)
+
+    def _add(self, h: torch.Tensor, branch) -> None:
+        if isinstance(branch, ScaledBranch):
+            ops.add_scaled_rmsnorm(h, branch.rows, branch.scale, self.weight, self.eps, None)
+        else:
+            ops.add_rmsnorm(h, [branch], self.weight, self.eps, None)
 
     def rms_prologue(self):
         return self.weight, self.eps
@@ -63,6 +70,20 @@ class RmsNorm(Part):
             ops.add_partials_rmsnorm(residual.h, slab, self.weight, self.eps, out)
             residual.pending = pending = []
             if rows is None:
+                return out
+        if any(isinstance(branch, ScaledBranch) for branch in pending):
+            # branches with a scale of their own: each is added by the kernel that knows the scale, the last one
+            # together with the norm
+            for branch in pending[:-1]:
+                self._add(residual.h, branch)
+            last = pending[-1]
+            if not isinstance(last, ScaledBranch):
+                pending = [last]
+            else:
+                count = residual.h.shape[0] if rows is None else rows.numel()
+                out = torch.empty((count, residual.h.shape[1]), dtype=self.build.dtype, device=residual.h.device)
+                ops.add_scaled_rmsnorm(residual.h, last.rows, last.scale, self.weight, self.eps, out, rows)
+                residual.pending = [] if rows is None else [last]
                 return out
         while len(pending) > 2:                    # more than two branches: add the extra ones first
             ops.add_rmsnorm(residual.h, pending[:2], self.weight, self.eps, None)

@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..weights.loader import Expect
 from .base import BuildContext, Part, register_part
 
 
@@ -16,9 +17,15 @@ class PositionEncoding(Part):
 
     An encoding that (also) biases the scores by distance sets ``score_slopes``: a float32 tensor [query heads]
     on the device, with score(head, query at s, key at p) -= score_slopes[head] * (s - p).  The attention part
-    then takes its general kernel, which knows the term; the matrix-core and fused decode kernels do not."""
+    then takes its general kernel, which knows the term; the matrix-core and fused decode kernels do not.
+    A bias that grows with the logarithm of the distance sets ``score_log_bias`` instead: float32 [query heads, 2]
+    = (r1, r2) with score -= r1 * ln(1 + r2 * (s - p)).  An encoding with tensors of its own sets ``learned``; it
+    then declares them (``expected_tensors(spec, prefix, hidden_size)``, beside the mixer's) and is built with
+    ``prefix`` and ``tensors``."""
     kernel_modules = ("attention",)
     score_slopes = None
+    score_log_bias = None
+    learned = False
 
     def fused_rotation(self):
         """What a kernel that rotates q and the new key itself has to apply in place of ``rotate_and_store``:
@@ -68,3 +75,23 @@ class Rope(PositionEncoding):
         ops.rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, step.positions, self.inv_freq,
                           self.rotary_dim, step.slot_mappings[cache.group] if owns else None,
                           cache.k_cache if owns else None, cache.v_cache if owns else None)
+
+
+@register_part("log_distance")
+class LogDistanceBias(PositionEncoding):
+    """No rotation of q and k: a key n positions behind the query loses r1[head] * ln(1 + r2[head] * n) of its
+    score, r1 and r2 learned numbers of each query head (tensors ``r1`` and ``r2`` beside the mixer's)."""
+    graph_safe = True
+    learned = True
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        return [Expect(f"{prefix}.r1", ((spec.num_heads,),), init="positive"),
+                Expect(f"{prefix}.r2", ((spec.num_heads,),), init="positive")]
+
+    def __init__(self, spec, head_dim: int, build: BuildContext, prefix: str = "", tensors=None):
+        pair = torch.stack([tensors[f"{prefix}.r1"].to(torch.float32), tensors[f"{prefix}.r2"].to(torch.float32)], dim=1)
+        self.score_log_bias = pair.contiguous().to(build.device)
+
+    def fused_rotation(self):
+        return None

@@ -52,12 +52,30 @@ class WeightError(ValueError):
 @dataclass(frozen=True)
 class Expect:
     """One tensor a part needs.  ``shapes[0]`` is the canonical shape (the one written by
-    the random-weights mode); the others are accepted on disk and reshaped to it.
-    ``init`` names the distribution used by the random-weights mode."""
+    the random-weights mode); the others are accepted on disk and reshaped to it.  A size of -1 in the
+    canonical shape stands for any size: the tensor's own shape gives it (``free_size`` is what the
+    random-weights mode writes there).  ``init`` names the distribution used by the random-weights mode.
+    ``optional``: the checkpoint may or may not hold it; it is handed out only if it does."""
     name: str
     shapes: Tuple[Tuple[int, ...], ...]
     init: str = "linear"
     integer: bool = False
+    optional: bool = False
+    free_size: int = 16
+
+    def accepts(self, shape) -> bool:
+        shape = tuple(shape)
+        for wanted in self.shapes:
+            if len(wanted) == len(shape) and all(w == -1 or w == s for w, s in zip(wanted, shape)):
+                return True
+        return False
+
+    def canonical(self, shape) -> Tuple[int, ...]:
+        """The canonical shape with its free sizes taken from a stored ``shape`` of as many dimensions."""
+        first = self.shapes[0]
+        if -1 not in first:
+            return first
+        return tuple(s if w == -1 else w for w, s in zip(first, shape))
 
 
 class WeightSource:
@@ -73,6 +91,19 @@ class WeightSource:
             for name in handle.names():
                 self._where[name] = handle
                 self._stored[name] = name
+
+    def apply_stored_names(self, stored_name, names: Sequence[str]) -> None:
+        """Let the tensors that an architecture's checkpoints store under names of their own answer to the
+        model's names: ``stored_name(name)`` is the stored spelling of each of the model's ``names``.  A stored
+        tensor that no name of the model stands for keeps its own name (and ``bind`` reports it)."""
+        renamed = dict(self._stored)
+        for name in names:
+            stored = stored_name(name)
+            if stored != name and stored in self._where and name not in renamed:
+                renamed[name] = stored
+                if renamed.get(stored) == stored:
+                    del renamed[stored]
+        self._stored = renamed
 
     def apply_aliases(self, aliases: Sequence[Tuple[str, str]], root_prefix: str = "") -> None:
         """Let tensors stored under another spelling answer to the model's names.  ``aliases``:
@@ -166,7 +197,7 @@ def bind(source: WeightSource, expectations: Sequence[Expect],
     for expect in expectations:
         wanted[expect.name] = expect                      # a name asked for twice (tied weights) is one tensor
     present = set(source.names())
-    missing = sorted(name for name in wanted if name not in present)
+    missing = sorted(name for name in wanted if name not in present and not wanted[name].optional)
     unexpected = []
     for name in sorted(present - set(wanted)):
         original = (copies or {}).get(name)
@@ -184,7 +215,7 @@ def bind(source: WeightSource, expectations: Sequence[Expect],
     for name, expect in wanted.items():
         if name not in present:
             continue
-        if tuple(source.shape(name)) not in expect.shapes:
+        if not expect.accepts(source.shape(name)):
             wrong_shape.append((name, expect.shapes, tuple(source.shape(name))))
         if not expect.integer and not source.dtype(name).is_floating_point:
             wrong_dtype.append((name, str(source.dtype(name))))
@@ -193,7 +224,11 @@ def bind(source: WeightSource, expectations: Sequence[Expect],
     out: Dict[str, torch.Tensor] = {}
     narrowed: List[str] = []
     for name, expect in wanted.items():
-        tensor = source.tensor(name).reshape(expect.shapes[0])
+        if name not in present:
+            continue                                       # an optional tensor the checkpoint does not hold
+        tensor = source.tensor(name)
+        tensor = tensor.reshape(expect.canonical(tensor.shape) if len(tensor.shape) == len(expect.shapes[0])
+                                else expect.shapes[0])
         if expect.integer:
             tensor = tensor.to(torch.int32)
         elif tensor.dtype == torch.float64:

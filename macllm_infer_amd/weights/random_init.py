@@ -44,7 +44,7 @@ def random_tensors(config, seed: int, storage_dtype: torch.dtype = torch.bfloat1
 
     out: Dict[str, torch.Tensor] = {}
     for expect in DecoderModel.expected_tensors(config.to_model_spec()):
-        shape = expect.shapes[0]
+        shape = tuple(expect.free_size if size == -1 else size for size in expect.shapes[0])
         kind = expect.init
         if kind == "linear":
             tensor = normal(shape, 1.0 / math.sqrt(shape[-1]) if unit else 0.02)
@@ -60,6 +60,14 @@ def random_tensors(config, seed: int, storage_dtype: torch.dtype = torch.bfloat1
             tensor = torch.log(uniform(shape, 1.0, 16.0))
         elif kind == "D":
             tensor = normal(shape, 0.1, 1.0)
+        elif kind == "zero_centred":                       # a weight stored as its distance from one
+            tensor = normal(shape, 0.1)
+        elif kind == "scale":                              # a scale on a branch, around one
+            tensor = normal(shape, 0.2, 1.0)
+        elif kind == "positive":                           # a positive rate
+            tensor = uniform(shape, 0.05, 1.5)
+        elif kind == "logit":                              # a number that enters an exponential or a sigmoid
+            tensor = normal(shape, 1.0)
         elif kind == "dt_bias":
             step = torch.exp(uniform(shape, math.log(1e-3), math.log(0.1)))
             tensor = step + torch.log(-torch.expm1(-step))          # inverse softplus
@@ -78,5 +86,9 @@ def write_random_model(config, seed: int, folder: str, storage_dtype: torch.dtyp
     raw["torch_dtype"] = "bfloat16" if storage_dtype == torch.bfloat16 else "float32"
     with open(os.path.join(folder, "config.json"), "w") as handle:
         json.dump(raw, handle, indent=1)
-    write_safetensors(os.path.join(folder, "model.safetensors"), random_tensors(config, seed, storage_dtype, preset))
+    spec = config.to_model_spec()
+    tensors = random_tensors(config, seed, storage_dtype, preset)
+    # under the names the architecture's checkpoints use
+    write_safetensors(os.path.join(folder, "model.safetensors"),
+                      {spec.stored_name(name): tensor for name, tensor in tensors.items()})
     return folder

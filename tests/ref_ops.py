@@ -85,13 +85,14 @@ def linear(x, weight, bias, keep_float32=False):
 
 
 def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, rotary_dim, slot_mapping,
-                  k_cache, v_cache):
+                  k_cache, v_cache, value_dim=None):
     T = qkv.shape[0]
+    value_dim = head_dim if value_dim is None else value_dim
     q_cols = num_heads * head_dim
     k_cols = num_kv_heads * head_dim
     q = _f(qkv[:, :q_cols]).reshape(T, num_heads, head_dim).clone()
     k = _f(qkv[:, q_cols:q_cols + k_cols]).reshape(T, num_kv_heads, head_dim).clone()
-    v = qkv[:, q_cols + k_cols:q_cols + 2 * k_cols].reshape(T, num_kv_heads, head_dim)
+    v = qkv[:, q_cols + k_cols:q_cols + k_cols + num_kv_heads * value_dim].reshape(T, num_kv_heads, value_dim)
     if inv_freq is not None and rotary_dim > 0:
         half = rotary_dim // 2
         angle = positions.to(torch.float32)[:, None] * inv_freq[None, :]
@@ -112,11 +113,13 @@ def rope_kv_store(qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, r
 
 def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_tables, lane_of_token,
                     positions, scale, window, out, max_seq_len=None, slopes=None, query_tiles=None, tile_tokens=0,
-                    cu_seqlens=None):
+                    cu_seqlens=None, log_bias=None, sinks=None, value_dim=None):
     """``max_seq_len`` sizes the kernel's launch and nothing else: not used here, and neither is the table of
     runs that picks the kernel for lanes of several tokens.  ``slopes``: a bias on the scores,
-    ``-slopes[head] * (query position - key position)``."""
+    ``-slopes[head] * (query position - key position)``; ``log_bias`` [Hq, 2] = (r1, r2): the scores lose
+    r1 * ln(1 + r2 * distance); ``sinks`` [Hq]: exp(sink) is one more term of the denominator."""
     T = q.shape[0]
+    value_dim = head_dim if value_dim is None else value_dim
     page_size = k_cache.shape[2]
     group = num_heads // num_kv_heads
     for token in range(T):
@@ -133,8 +136,13 @@ def paged_attention(q, num_heads, num_kv_heads, head_dim, k_cache, v_cache, bloc
             scores = (k[:, head // group, :] @ query) * scale
             if slopes is not None:
                 scores = scores - slopes[head] * (position - keys).float()
-            weights = torch.softmax(scores, dim=0)
-            out[token, head * head_dim:(head + 1) * head_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
+            if log_bias is not None:
+                scores = scores - log_bias[head, 0] * torch.log1p(log_bias[head, 1] * (position - keys).float())
+            if sinks is not None:
+                weights = torch.softmax(torch.cat([scores, sinks[head].reshape(1)]), dim=0)[:-1]
+            else:
+                weights = torch.softmax(scores, dim=0)
+            out[token, head * value_dim:(head + 1) * value_dim] = (weights @ v[:, head // group, :]).to(out.dtype)
 
 
 def decode_attention_supported(dtype, num_heads, num_kv_heads, head_dim, page_size):
@@ -216,12 +224,84 @@ def gate_norm(y, z, weight, num_groups, eps, out):
     out.copy_(v.to(out.dtype))
 
 
+def add_scaled_rmsnorm(h, delta, scale, weight, eps, out, rows=None):
+    total = h + _f(delta) * scale
+    if rows is None:
+        h.copy_(total)
+        picked = total
+    else:
+        picked = total[rows.long()]
+    if out is not None:
+        out.copy_((picked / torch.sqrt(picked.pow(2).mean(-1, keepdim=True) + eps) * weight).to(out.dtype))
+
+
+def polynorm(z, coefficients, eps, out):
+    x = _f(z)
+    unit = lambda values: values / torch.sqrt(values.pow(2).mean(-1, keepdim=True) + eps)
+    c = coefficients
+    out.copy_((c[0] * unit(x) + c[1] * unit(x * x) + c[2] * unit(x * x * x) + c[3]).to(out.dtype))
+
+
+def tanh_rows(x, out):
+    out.copy_(torch.tanh(_f(x)).to(out.dtype))
+
+
+def head_norm_gate(raw, gate, weight, num_heads, eps, activation, out):
+    T, width = raw.shape
+    heads = raw.reshape(T, num_heads, width // num_heads)
+    normed = (heads / torch.sqrt(heads.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, width)
+    if weight is not None:
+        normed = normed * weight
+    g = _f(gate)
+    out.copy_((normed * (F.silu(g) if activation == "silu" else torch.sigmoid(g))).to(out.dtype))
+
+
+def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, state, cu_seqlens, slot_ids, out,
+                      max_query_len=0, head_decay=None, key_scale=1.0, positions=None, inv_freq=None, rotary_dim=0,
+                      removal_col=-1, decay_logits=None, decay_bias=None, decay_floor=0.0, key_eps=0.0):
+    """``state`` [slots, H, value dim, key dim] holds the transposed state of every head."""
+    H, K, V = num_heads, key_dim, value_dim
+    T = u.shape[0]
+    q = _f(u[:, q_col:q_col + H * K]).reshape(T, H, K).clone()
+    k = _f(u[:, k_col:k_col + H * K]).reshape(T, H, K).clone()
+    v = _f(u[:, v_col:v_col + H * V]).reshape(T, H, V)
+    delta = removal_col >= 0
+    if inv_freq is not None and rotary_dim > 0:
+        half = rotary_dim // 2
+        angle = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+        cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+
+        def rotate(x):
+            a, b = x[..., :half], x[..., half:rotary_dim]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., rotary_dim:]], dim=-1)
+        q, k = rotate(q), rotate(k)
+    if delta:
+        unit = k / torch.sqrt(k.pow(2).sum(-1, keepdim=True) + key_eps)
+        removal = torch.sigmoid(_f(u[:, removal_col:removal_col + H * K])).reshape(T, H, K)
+        decay = torch.exp(-decay_floor * torch.sigmoid(decay_logits + decay_bias)).reshape(T, H, K)
+    else:
+        k = k * key_scale
+    for lane in range(cu_seqlens.numel() - 1):
+        slot = int(slot_ids[lane])
+        S = state[slot].transpose(-1, -2).clone()                   # [H, K, V]
+        for t in range(int(cu_seqlens[lane]), int(cu_seqlens[lane + 1])):
+            if delta:
+                along = torch.einsum("hk,hkv->hv", unit[t], S)
+                S = decay[t][:, :, None] * S - (removal[t] * unit[t])[:, :, None] * along[:, None, :] \
+                    + k[t][:, :, None] * v[t][:, None, :]
+            else:
+                S = head_decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, q[t]).reshape(H * V)
+        state[slot] = S.transpose(-1, -2)
+
+
 def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
 NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "tanh_softcap", "linear", "rope_kv_store", "paged_attention",
-         "conv1d_silu", "conv_state_update", "conv_step", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed"]
+         "conv1d_silu", "conv_state_update", "conv_step", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed",
+         "add_scaled_rmsnorm", "polynorm", "tanh_rows", "head_norm_gate", "linear_state_scan"]
 
 
 def install(monkeypatch):
