@@ -4,6 +4,7 @@ MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
     python bench.py --workload serving [--shape 0.5b|7b|34b]
     python bench.py --microbench
+    python bench.py --design mukutar [--shape 0.5b|7b] [--layers L] [--window W] [--only mukutar|falcon_h1]
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
@@ -23,6 +24,13 @@ over K; then the skinny kernel's tiles of 16 features).
 
 ``--microbench`` prints what this GPU's memory delivers to a plain streaming read and a plain
 read-modify-write (the ceilings that the decode kernels can be held against).
+
+``--design mukutar`` measures a Mukutar-shaped model (layers in turn: windowed attention with a logarithmic
+distance bias and a sink, generalized delta rule, retention; PolyNorm feed-forwards; random weights) whose
+sizes are those of ``--shape``, and beside it the Falcon-H1 shape with the same width, layer count, heads and
+feed-forward width: for both the 2,048-token prompt step and decode steps at batch 1, 8 and 64 behind
+2,048-token contexts, each with its fraction of the peak (prompt: flops; decode: bytes the step has to read).
+The default workload and its line are not touched by it.
 
 ``--workload serving`` runs whole requests through the scheduler and the sampler instead
 (``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
@@ -121,6 +129,125 @@ def serving(args, shape) -> int:
     return 0
 
 
+def mukutar_shape(shape: dict, layers: int, window: int) -> dict:
+    """A Mukutar configuration with the sizes of a Falcon-H1 ``shape``: the same width, vocabulary, feed-forward
+    width, attention heads and head size; the recurrent mixers as wide as the stream."""
+    width, dim = shape["hidden_size"], shape["head_dim"]
+    attention = {"type": "attention", "mixer": {
+        "heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"], "dim": dim, "vdim": dim,
+        "scale": dim ** -0.5, "mask": {"size": window}}}
+    delta_heads = width // dim
+    general_delta = {"type": "general_delta", "mixer": {"heads": delta_heads, "dim": dim, "decay_rank": 64}}
+    retention_heads = max(width // (2 * dim), 1)
+    retention = {"type": "retention", "mixer": {
+        "heads": retention_heads, "dim": dim, "vdim": 2 * dim, "rot": {"base": 1e6, "dims": dim},
+        "decay": [1.0 - 2.0 ** (-5.0 - 4.0 * head / max(retention_heads - 1, 1)) for head in range(retention_heads)]}}
+    kinds = (attention, general_delta, retention)
+    mlp = {"kind": "dense", "ff": shape["intermediate_size"]}
+    return {"architecture": "Mukutar", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
+            "layers": [dict(kinds[index % 3], mlp=mlp) for index in range(layers)]}
+
+
+def design_points(args) -> int:
+    """Prompt and decode steps of a Mukutar-shaped model and of the Falcon-H1 shape of equal sizes."""
+    import torch
+    from macllm_infer_amd import Engine, Lane
+    from macllm_infer_amd.config import FalconH1Config, MukutarConfig
+    from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
+    from macllm_infer_amd.weights.random_init import random_tensors
+
+    shape = SHAPES[args.shape]
+    layers = args.layers or 12
+    storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    element = 2 if args.dtype == "bf16" else 4
+    configs = {"mukutar": MukutarConfig.from_dict(mukutar_shape(shape, layers, args.window)),
+               "falcon_h1": FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))}
+    batches = [] if args.prefill_only else ([args.batch] if args.skip_points else sorted({1, args.batch, 64}))
+    largest = max(batches, default=1)
+    per_request = -(-(CONTEXT + args.steps + args.warmup + 1) // 64) * 64
+    out = {}
+    for name, config in configs.items():
+        if args.only and name != args.only:
+            continue
+        tensors = random_tensors(config, 0, storage, "baseline", device="cuda:0")
+        engine = Engine(config=config, tensors=tensors, dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                        kv_cache_block_tokens=args.page_tokens,
+                        kv_cache_capacity_tokens=per_request * largest + PREFILL_TOKENS + 64,
+                        max_active_sequences=largest + 1, measured_paths=not args.fixed_paths)
+        parameters = sum(tensor.numel() for tensor in tensors.values())
+        del tensors
+        sampler = Sampler(engine.vocab_size, engine.device)
+        generator = torch.Generator().manual_seed(0)
+        vocab = engine.vocab_size
+
+        def prefill_step():
+            prompt = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=generator).tolist()
+            engine.add_request("prefill")
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            engine.step([Lane("prefill", prompt, [PREFILL_TOKENS - 1])])
+            torch.cuda.synchronize()
+            seconds = time.perf_counter() - started
+            engine.finish("prefill")
+            return seconds
+
+        times = [prefill_step() for _ in range(6)]
+        seconds = sorted(times[3:])[1]
+        flops = total(prefill_costs(engine.spec, PREFILL_TOKENS, element)).flops
+        record = {"parameters_m": round(parameters / 1e6, 1),
+                  "prefill": {"value": round(PREFILL_TOKENS / seconds, 1), "ms": round(seconds * 1e3, 3),
+                              "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 5)}}
+        for batch in batches:
+            names = [f"b{batch}_{index}" for index in range(batch)]
+            for request in names:
+                engine.add_request(request)
+                engine.step([Lane(request, torch.randint(0, vocab, (CONTEXT,), generator=generator).tolist(), [])])
+            rows = [SamplerRow(GREEDY, (), ()) for _ in names]
+            tokens = torch.randint(0, vocab, (batch,), generator=generator).tolist()
+
+            def decode_step(before):
+                if before is None:
+                    lanes = [Lane(request, [token], [0]) for request, token in zip(names, tokens)]
+                else:
+                    lanes = [Lane(request, [0], [0], feed=(before.device, row)) for row, request in enumerate(names)]
+                return sampler.sample_async(engine.step(lanes), rows)
+
+            on_their_way = decode_step(None)
+            for _ in range(args.warmup):
+                newer = decode_step(on_their_way)
+                on_their_way.wait()
+                on_their_way = newer
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            for _ in range(args.steps):
+                newer = decode_step(on_their_way)
+                on_their_way.wait()
+                on_their_way = newer
+            torch.cuda.synchronize()
+            step_seconds = (time.perf_counter() - started) / args.steps
+            for request in names:
+                engine.finish(request)
+            moved = total(decode_step_costs(engine.spec, batch, CONTEXT + args.warmup + args.steps / 2.0, element))
+            record[f"decode_b{batch}"] = {"value": round(batch / step_seconds, 1), "ms": round(step_seconds * 1e3, 4),
+                                          "read_mb": round(moved.read / 1e6, 1),
+                                          "frac": round(moved.read / step_seconds / PEAK_HBM_BYTES, 5)}
+        out[name] = record
+        del engine, sampler
+        torch.cuda.empty_cache()
+    first = out.get("mukutar") or next(iter(out.values()))
+    headline = first.get(f"decode_b{args.batch}", first["prefill"])
+    print(json.dumps({
+        "metric": "Mukutar-shaped model beside the Falcon-H1 shape of equal sizes: prefill tok/s at 2,048 tokens, "
+                  "decode tok/s at batch 1 / 8 / 64 behind 2,048-token contexts",
+        "value": headline["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "dtype": args.dtype, "data": "synthetic",
+        "config": {"shape": args.shape, "layers": layers, "hidden": shape["hidden_size"],
+                   "intermediate": shape["intermediate_size"], "head_dim": shape["head_dim"], "window": args.window,
+                   "vocab": shape["vocab_size"], "seq_len": CONTEXT, "page_tokens": args.page_tokens},
+        "models": out}))
+    return 0
+
+
 def microbench() -> int:
     """Streaming read and read-modify-write bandwidth of this GPU, with this package's own kernels."""
     import torch
@@ -186,6 +313,11 @@ def main() -> int:
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     parser.add_argument("--microbench", action="store_true",
                         help="only this GPU's streaming read and read-modify-write bandwidth")
+    parser.add_argument("--design", default=None, choices=["mukutar"],
+                        help="measure a model of this design with the sizes of --shape (12 layers unless --layers) beside "
+                             "the Falcon-H1 shape of equal sizes, instead of the headline workload")
+    parser.add_argument("--window", type=int, default=1024, help="--design: the attention layers' window")
+    parser.add_argument("--only", default=None, choices=["mukutar", "falcon_h1"], help="--design: one of the two models")
     parser.add_argument("--write-config", default=None, metavar="PATH",
                         help="write the config.json of --shape / --layers there and exit (what "
                              "utils.kernel_trace --config reads)")
@@ -198,8 +330,14 @@ def main() -> int:
     if args.write_config:
         shape = SHAPES[args.shape]
         with open(args.write_config, "w") as handle:
-            json.dump(dict(shape, num_hidden_layers=args.layers or shape["num_hidden_layers"]), handle)
+            if args.design == "mukutar" and args.only != "falcon_h1":
+                json.dump(mukutar_shape(shape, args.layers or 12, args.window), handle)
+            else:
+                layers = args.layers or (12 if args.design else shape["num_hidden_layers"])
+                json.dump(dict(shape, num_hidden_layers=layers), handle)
         return 0
+    if args.design:
+        return design_points(args)
     if args.workload == "serving":
         return serving(args, SHAPES[args.shape])
 

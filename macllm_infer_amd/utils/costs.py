@@ -36,19 +36,39 @@ def model_sizes(spec) -> dict:
     d = spec.hidden_size
     total = dict(in_weights=0, out_weights=0, gate_up=0, down=0, kv_per_token=0, state=0, conv_tail=0,
                  attention=0, scan=0, layers=len(spec.schedule), head=spec.vocab_size * d, hidden=d,
-                 mixed=0, inner=0, in_width=0)
+                 mixed=0, inner=0, in_width=0, windows=[], linear_scan=0)
     for entry in spec.schedule:
         layer = spec.layers[entry.layer]
         for slot in layer.mixers:
             part = slot.spec
             if part.kind == "attention":
                 q, kv = part.num_heads * part.head_dim, part.num_kv_heads * part.head_dim
-                total["in_weights"] += (q + 2 * kv) * d
-                total["out_weights"] += d * q
-                total["kv_per_token"] += 2 * kv if entry.kv_from is None else 0
-                total["attention"] += part.num_heads * part.head_dim      # x 2 T^2 flops (causal: half of 4 T^2)
-                total["mixed"] += q
-                total["in_width"] += q + 2 * kv
+                values, mixed = part.num_kv_heads * part.value_width, part.num_heads * part.value_width
+                total["in_weights"] += (q + kv + values) * d
+                total["out_weights"] += d * mixed
+                total["kv_per_token"] += kv + values if entry.kv_from is None else 0
+                # x 2 T^2 flops (causal: half of 4 T^2); a window w keeps min(i + 1, w) keys for the query at i
+                total["attention"] += part.num_heads * (part.head_dim + part.value_width) / 2.0
+                total["windows"].append((part.num_heads * (part.head_dim + part.value_width) / 2.0,
+                                         (kv + values) if entry.kv_from is None else 0, part.window))
+                total["mixed"] += mixed
+                total["in_width"] += q + kv + values
+            elif part.kind == "retention":
+                keys, values = part.num_heads * part.key_dim, part.num_heads * part.value_dim
+                total["in_weights"] += (2 * keys + 2 * values) * d
+                total["out_weights"] += d * values
+                total["state"] += part.num_heads * part.key_dim * part.value_dim
+                total["linear_scan"] += 4 * part.num_heads * part.key_dim * part.value_dim     # x T flops
+                total["mixed"] += values
+                total["in_width"] += 2 * keys + 2 * values
+            elif part.kind == "general_delta":
+                inner, rank = part.num_heads * part.head_dim, part.decay_rank or 0
+                total["in_weights"] += (5 * inner + rank) * d + inner * rank
+                total["out_weights"] += d * inner
+                total["state"] += part.num_heads * part.head_dim ** 2
+                total["linear_scan"] += 10 * part.num_heads * part.head_dim ** 2               # x T flops
+                total["mixed"] += inner
+                total["in_width"] += 5 * inner + rank
             elif part.kind == "mamba2":
                 total["in_weights"] += part.projection_width * d
                 total["out_weights"] += d * part.inner_size
@@ -57,22 +77,38 @@ def model_sizes(spec) -> dict:
                 total["scan"] += part.num_heads * part.head_dim * part.state_size      # x 6 T flops
                 total["mixed"] += part.inner_size
                 total["in_width"] += part.projection_width
+        if layer.ffn is None:
+            continue
         if layer.ffn.kind == "swiglu":
             total["gate_up"] += 2 * layer.ffn.intermediate_size * d
             total["down"] += d * layer.ffn.intermediate_size
             total["inner"] += layer.ffn.intermediate_size
+        elif layer.ffn.kind == "polynorm_ffn":
+            total["gate_up"] += layer.ffn.intermediate_size * d
+            total["down"] += d * layer.ffn.intermediate_size
+            total["inner"] += layer.ffn.intermediate_size
     return total
+
+
+def keys_seen(tokens: float, window) -> float:
+    """Sum over the queries 0 .. tokens-1 of one prompt of the keys each sees: min(i + 1, window)."""
+    if not window or window >= tokens:
+        return tokens * (tokens + 1) / 2.0
+    return window * (window + 1) / 2.0 + (tokens - window) * window
 
 
 def decode_step_costs(spec, batch: int, context: float, element: int = 2) -> Dict[str, Cost]:
     """A step of ``batch`` single tokens whose requests hold ``context`` tokens each."""
     s = model_sizes(spec)
     rows = batch
+    kept = lambda window: min(context, window) if window else context          # keys a query still sees
+    kv_read = sum(per_token * kept(window) for _, per_token, window in s["windows"])
+    attention_flops = sum(4.0 * width * kept(window) for width, _, window in s["windows"])
     return {
         "input projections": Cost(s["in_weights"] * element, 0, 2.0 * rows * s["in_weights"]),
-        "mixers": Cost(batch * (s["kv_per_token"] * context * element + s["state"] * 4 + s["conv_tail"] * element),
+        "mixers": Cost(batch * (kv_read * element + s["state"] * 4 + s["conv_tail"] * element),
                        batch * (s["kv_per_token"] * element + s["state"] * 4 + s["conv_tail"] * element),
-                       batch * (2.0 * s["attention"] * 2 * context + 6.0 * s["scan"])),
+                       batch * (attention_flops + 6.0 * s["scan"] + s["linear_scan"])),
         "output projections": Cost(s["out_weights"] * element, 0, 2.0 * rows * s["out_weights"]),
         "gate and up projections": Cost(s["gate_up"] * element, 0, 2.0 * rows * s["gate_up"]),
         "down projections": Cost(s["down"] * element, 0, 2.0 * rows * s["down"]),
@@ -88,8 +124,9 @@ def prefill_costs(spec, tokens: int, element: int = 2) -> Dict[str, Cost]:
     rows_moved = T * element * (s["hidden"] * 4 * s["layers"] + s["in_width"] + s["mixed"] + 3 * s["inner"])
     return {
         "matrix products": Cost(weights * element + rows_moved, 0, 2.0 * T * weights + 2.0 * s["head"]),
-        "attention": Cost(T * s["kv_per_token"] * element, T * s["kv_per_token"] * element, 2.0 * s["attention"] * T * T),
-        "state-space scan": Cost(s["state"] * 4, s["state"] * 4, 6.0 * s["scan"] * T),
+        "attention": Cost(T * s["kv_per_token"] * element, T * s["kv_per_token"] * element,
+                          sum(4.0 * width * keys_seen(T, window) for width, _, window in s["windows"])),
+        "state-space scan": Cost(s["state"] * 4, s["state"] * 4, 6.0 * s["scan"] * T + s["linear_scan"] * T),
     }
 
 
@@ -109,7 +146,7 @@ def total(costs: Dict[str, Cost]) -> Cost:
 DECODE_GROUPS: List[Tuple[str, str]] = [
     (r"mixer_decode_kernel|mixer_merge_kernel|decode_attention_kernel|decode_merge_kernel|ssm_scan_kernel|conv_step_kernel|"
      r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel|paged_attention_tile_kernel|"
-     r"paged_attention_merge_kernel", "mixers"),
+     r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel", "mixers"),
     (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
     (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
     (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
@@ -120,7 +157,8 @@ PREFILL_GROUPS: List[Tuple[str, str]] = [
     (r"^Cijk_|gemm_f32_kernel", "matrix products"),
     (r"prefill_attention|paged_attention_kernel|paged_attention_tile_kernel|paged_attention_merge_kernel|"
      r"rope_kv_store_kernel", "attention"),
-    (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel", "state-space scan"),
+    (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel|linear_state_|head_norm_gate_kernel|"
+     r"tanh_rows_kernel", "state-space scan"),
 ]
 
 
