@@ -19,7 +19,17 @@
 // takes (lane of the step, head, a run of columns) and walks the lane's tokens in order; the per-token vectors
 // (q, k, and for the delta rule w, u, a*u) are laid in LDS for a stage of tokens at a time by the waves of the
 // workgroup, one token a wave at a time, and read from there by every column.  R and the order of every sum depend
-// on dk alone, so a token's result is the same bits however the step is cut and whatever else it holds.
+// on dk alone.
+//
+// Long portions run in three passes over chunks of the lanes (a table of (lane, first row, tokens, index in the
+// lane) that the step carries), so that the tokens of one prompt are worked on side by side:
+//   local   every chunk but a lane's last, from an empty state: the state B the chunk's own tokens leave, and for
+//           the delta rule the chunk's transition P = A_last ... A_first (A_t = diag(w_t) - (a_t u_t) u_t^T), whose
+//           column i is what the same recurrence without keys makes of the unit vector e_i: dk more columns;
+//   carry   per lane, chunk after chunk: S_start(c + 1) = P_c S_start(c) + B_c (retention: P_c = decay^tokens),
+//           beginning with the request's state; every chunk's starting state is kept;
+//   scan    every chunk from its starting state: the outputs, and behind a lane's last chunk the state of the request.
+// All of it in float32: the passes add the same products in another order.
 #include "common.h"
 
 #define LS_MAX_PER_LANE 16          // key channels of a column that one lane keeps
@@ -47,7 +57,15 @@ struct ScanArgs {
   const float* decay_bias;          // [H * dk]
   float decay_floor, key_eps;
   int R, per_lane, columns, stage;  // lanes a column, key channels a lane, columns a workgroup, tokens a stage
+  const int* chunks;                // passes over chunks: [chunks, 4] = (lane, first row, tokens, index in the lane)
+  const int* lane_chunks;           // [lanes, 2] = (first chunk, chunks)
+  float* local;                     // [chunks, H, dv (+ dk), dk]: what the local pass leaves
+  float* start;                     // [chunks, H, dv, dk]: every chunk's starting state
 };
+
+#define LS_WHOLE 0                  // a lane from and into its request's state
+#define LS_LOCAL 1                  // a chunk from an empty state (and the unit vectors): no outputs
+#define LS_CHUNK 2                  // a chunk from its starting state
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
@@ -57,14 +75,26 @@ __device__ __forceinline__ float column_sum(float v, int R) {
   return v;
 }
 
-template <typename T, bool DELTA>
+template <typename T, bool DELTA, int MODE>
 __global__ void __launch_bounds__(LS_THREADS)
 linear_state_scan_kernel(const ScanArgs a) {
   extern __shared__ __align__(16) float stage_lds[];
-  const int lane_of_step = blockIdx.x;
   const int head = blockIdx.y;
-  const int first_token = a.cu_seqlens[lane_of_step];
-  const int end_token = a.cu_seqlens[lane_of_step + 1];
+  int lane_of_step, first_token, end_token;
+  bool last_of_lane = true;
+  if (MODE == LS_WHOLE) {
+    lane_of_step = blockIdx.x;
+    first_token = a.cu_seqlens[lane_of_step];
+    end_token = a.cu_seqlens[lane_of_step + 1];
+  } else {
+    const int* row = a.chunks + 4 * blockIdx.x;
+    lane_of_step = row[0];
+    if (lane_of_step < 0) return;                          // a row past the step's own chunks
+    first_token = row[1];
+    end_token = first_token + row[2];
+    last_of_lane = row[3] == a.lane_chunks[2 * lane_of_step + 1] - 1;
+    if (MODE == LS_LOCAL && last_of_lane) return;          // nothing follows it
+  }
   if (end_token <= first_token) return;
   const int tid = threadIdx.x;
   const int wave = tid / WAVE;
@@ -78,17 +108,23 @@ linear_state_scan_kernel(const ScanArgs a) {
   const int column_in_group = tid / R;
   const int sub = tid - column_in_group * R;
   const int column = blockIdx.z * a.columns + column_in_group;
-  const bool mine = column_in_group < a.columns && column < dv;
+  // the local pass of the delta rule carries dk more columns: the transition's, which start as the unit vectors
+  const int total_columns = (MODE == LS_LOCAL && DELTA) ? dv + dk : dv;
+  const bool mine = column_in_group < a.columns && column < total_columns;
   const int channel0 = sub * per_lane;
   const T* rows = (const T*)a.u;
 
   // the column's share of the state
   float s[LS_MAX_PER_LANE];
-  float* state_column = a.state + (((long)a.slot_ids[lane_of_step] * a.H + head) * dv + (mine ? column : 0)) * dk;
+  float* state_column = a.state + (((long)a.slot_ids[lane_of_step] * a.H + head) * dv + (mine && column < dv ? column : 0)) * dk;
+  const float* from = state_column;
+  if (MODE == LS_CHUNK) from = a.start + (((long)blockIdx.x * a.H + head) * dv + (mine ? column : 0)) * dk;
 #pragma unroll
   for (int e = 0; e < LS_MAX_PER_LANE; ++e) {
     const int channel = channel0 + e;
-    s[e] = (mine && e < per_lane && channel < dk) ? state_column[channel] : 0.f;
+    const bool held = mine && e < per_lane && channel < dk;
+    if (MODE == LS_LOCAL) s[e] = (held && channel == column - dv) ? 1.f : 0.f;
+    else s[e] = held ? from[channel] : 0.f;
   }
   const float decay = DELTA ? 0.f : a.head_decay[head];
   const int half = a.rotary_dim / 2;
@@ -177,26 +213,103 @@ linear_state_scan_kernel(const ScanArgs a) {
           for (int e = 0; e < LS_MAX_PER_LANE; ++e)
             if (e < per_lane) {
               s[e] = fmaf(k_lds[e], value, fmaf(-au_lds[e], along, w_lds[e] * s[e]));
-              result = fmaf(s[e], q_lds[e], result);
+              if (MODE != LS_LOCAL) result = fmaf(s[e], q_lds[e], result);
             }
         } else {
 #pragma unroll
           for (int e = 0; e < LS_MAX_PER_LANE; ++e)
             if (e < per_lane) {
               s[e] = fmaf(k_lds[e], value, decay * s[e]);
-              result = fmaf(s[e], q_lds[e], result);
+              if (MODE != LS_LOCAL) result = fmaf(s[e], q_lds[e], result);
             }
         }
-        result = column_sum(result, R);
-        if (mine && sub == 0) a.out[(long)(stage_first + tt) * a.out_ld + head * dv + column] = result;
+        if (MODE != LS_LOCAL) {
+          result = column_sum(result, R);
+          if (mine && sub == 0) a.out[(long)(stage_first + tt) * a.out_ld + head * dv + column] = result;
+        }
       }
     }
   }
-  if (mine) {
+  float* into = state_column;
+  if (MODE == LS_LOCAL) into = a.local + (((long)blockIdx.x * a.H + head) * total_columns + (mine ? column : 0)) * dk;
+  if (mine && (MODE != LS_CHUNK || last_of_lane)) {
 #pragma unroll
     for (int e = 0; e < LS_MAX_PER_LANE; ++e) {
       const int channel = channel0 + e;
-      if (e < per_lane && channel < dk) state_column[channel] = s[e];
+      if (e < per_lane && channel < dk) into[channel] = s[e];
+    }
+  }
+}
+
+// ---------------------------------------------------------------- the carry from chunk to chunk
+// One workgroup a (lane, head, run of LS_CARRY_COLUMNS value columns): the columns' states sit in LDS, a thread
+// owns key channels m and computes, for its columns j, s_j[m] <- sum_i P[m, i] s_j[i] + B_j[m] chunk after chunk
+// (P's column i is row dv + i of what the local pass left); every chunk's starting state goes to ``start``.
+#define LS_CARRY_COLUMNS 8
+
+template <bool DELTA>
+__global__ void __launch_bounds__(LS_THREADS)
+linear_state_carry_kernel(const ScanArgs a) {
+  extern __shared__ __align__(16) float carry_lds[];       // [LS_CARRY_COLUMNS][dk]
+  const int lane_of_step = blockIdx.x;
+  const int head = blockIdx.y;
+  const int first_chunk = a.lane_chunks[2 * lane_of_step];
+  const int count = a.lane_chunks[2 * lane_of_step + 1];
+  if (count <= 0) return;
+  const int dk = a.dk, dv = a.dv;
+  const int column0 = blockIdx.z * LS_CARRY_COLUMNS;
+  const int total_columns = DELTA ? dv + dk : dv;
+  const float* state = a.state + ((long)a.slot_ids[lane_of_step] * a.H + head) * dv * dk;
+  for (int index = threadIdx.x; index < LS_CARRY_COLUMNS * dk; index += blockDim.x) {
+    const int c = index / dk, m = index - c * dk;
+    const float value = column0 + c < dv ? state[(long)(column0 + c) * dk + m] : 0.f;
+    carry_lds[index] = value;
+    if (column0 + c < dv) a.start[(((long)first_chunk * a.H + head) * dv + column0 + c) * dk + m] = value;
+  }
+  __syncthreads();
+  const float decay = DELTA ? 0.f : a.head_decay[head];
+  for (int chunk = first_chunk; chunk < first_chunk + count - 1; ++chunk) {
+    const float* local = a.local + ((long)chunk * a.H + head) * total_columns * dk;
+    float* start = a.start + ((long)(chunk + 1) * a.H + head) * dv * dk;
+    const float shrink = DELTA ? 0.f : powf(decay, (float)a.chunks[4 * chunk + 2]);
+    // more key channels than threads: rounds of blockDim.x channels (the new values wait in registers of the round)
+    for (int m0 = 0; m0 < dk; m0 += blockDim.x) {
+      const int m = m0 + threadIdx.x;
+      float next[LS_CARRY_COLUMNS];
+#pragma unroll
+      for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = 0.f;
+      if (m < dk) {
+        if (DELTA) {
+          const float* transition = local + (long)dv * dk + m;       // P[m, i] at transition[i * dk]
+          for (int i = 0; i < dk; ++i) {
+            const float p = transition[(long)i * dk];
+#pragma unroll
+            for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = fmaf(p, carry_lds[c * dk + i], next[c]);
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = shrink * carry_lds[c * dk + m];
+        }
+#pragma unroll
+        for (int c = 0; c < LS_CARRY_COLUMNS; ++c)
+          if (column0 + c < dv) next[c] += local[(long)(column0 + c) * dk + m];
+      }
+      __syncthreads();                                      // the old state is read before any of it is replaced
+      if (m < dk) {
+#pragma unroll
+        for (int c = 0; c < LS_CARRY_COLUMNS; ++c) {
+          if (dk <= (int)blockDim.x) carry_lds[c * dk + m] = next[c];
+          if (column0 + c < dv) start[(long)(column0 + c) * dk + m] = next[c];
+        }
+      }
+    }
+    __syncthreads();
+    if (dk > (int)blockDim.x) {                             // several rounds: the new state comes back from memory
+      for (int index = threadIdx.x; index < LS_CARRY_COLUMNS * dk; index += blockDim.x) {
+        const int c = index / dk, m = index - c * dk;
+        carry_lds[index] = column0 + c < dv ? start[(long)(column0 + c) * dk + m] : 0.f;
+      }
+      __syncthreads();
     }
   }
 }
@@ -204,12 +317,11 @@ linear_state_scan_kernel(const ScanArgs a) {
 // How a head's state is dealt out: R lanes a column (the smallest power of two that leaves a lane at most
 // LS_MAX_PER_LANE key channels), per_lane = ceil(dk / R) channels a lane, LS_THREADS / R columns a workgroup of a
 // prompt portion (one wave's worth, 64 / R, for steps of single tokens, which want many small workgroups).
-extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col, int k_col, int v_col, int removal_col,
-                                    int H, int dk, int dv, float* state, const int* cu_seqlens, const int* slot_ids,
-                                    int lanes, float* out, long out_ld, int max_query_len, const float* head_decay,
-                                    float key_scale, const int* positions, const float* inv_freq, int rotary_dim,
-                                    const float* decay_logits, long logits_ld, const float* decay_bias,
-                                    float decay_floor, float key_eps, hipStream_t stream) {
+static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, int v_col, int removal_col, int H, int dk,
+                     int dv, float* state, const int* cu_seqlens, const int* slot_ids, int lanes, float* out, long out_ld,
+                     const float* head_decay, float key_scale, const int* positions, const float* inv_freq,
+                     int rotary_dim, const float* decay_logits, long logits_ld, const float* decay_bias,
+                     float decay_floor, float key_eps) {
   if (!u || !state || !cu_seqlens || !slot_ids || !out || lanes <= 0 || H <= 0 || dk <= 0 || dv <= 0)
     return ERR_BAD_ARGUMENT;
   const bool delta = removal_col >= 0;
@@ -218,34 +330,115 @@ extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col
   if (inv_freq && (!positions || rotary_dim <= 0 || rotary_dim > dk || (rotary_dim & 1))) return ERR_BAD_ARGUMENT;
   if (out_ld < (long)H * dv) return ERR_BAD_ARGUMENT;
   if (dk > LS_MAX_PER_LANE * WAVE || H > 65535 || lanes > 0x7fffffff) return ERR_UNSUPPORTED_SIZE;
-  ScanArgs a;
   a.u = u; a.ld = ld; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.removal_col = removal_col;
   a.H = H; a.dk = dk; a.dv = dv; a.state = state; a.cu_seqlens = cu_seqlens; a.slot_ids = slot_ids;
   a.out = out; a.out_ld = out_ld; a.head_decay = head_decay; a.key_scale = key_scale; a.positions = positions;
   a.inv_freq = inv_freq; a.rotary_dim = inv_freq ? rotary_dim : 0; a.decay_logits = decay_logits;
   a.logits_ld = logits_ld; a.decay_bias = decay_bias; a.decay_floor = decay_floor; a.key_eps = key_eps;
+  a.chunks = nullptr; a.lane_chunks = nullptr; a.local = nullptr; a.start = nullptr;
   int R = 1;
   while (R * LS_MAX_PER_LANE < dk) R *= 2;
   a.R = R;
   a.per_lane = (dk + R - 1) / R;
-  const int threads = max_query_len == 1 ? WAVE : LS_THREADS;
-  a.columns = threads / R;
-  if (a.columns > dv) a.columns = dv;
-  const int splits = (dv + a.columns - 1) / a.columns;
-  if (splits > 65535) return ERR_UNSUPPORTED_SIZE;
-  const int token_floats = (delta ? 5 : 2) * R * a.per_lane + a.columns;
+  return 0;
+}
+
+// columns a workgroup of ``threads`` threads takes of ``total_columns``, the tokens of a stage and its bytes in LDS
+static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, int longest, size_t* lds, int* splits) {
+  a.columns = threads / a.R;
+  if (a.columns > total_columns) a.columns = total_columns;
+  *splits = (total_columns + a.columns - 1) / a.columns;
+  if (*splits > 65535) return ERR_UNSUPPORTED_SIZE;
+  const int token_floats = (delta ? 5 : 2) * a.R * a.per_lane + a.columns;
   int stage = LS_STAGE_BYTES / (token_floats * (int)sizeof(float));
   if (stage > LS_STAGE_MOST) stage = LS_STAGE_MOST;
-  if (max_query_len > 0 && stage > max_query_len) stage = max_query_len;
+  if (longest > 0 && stage > longest) stage = longest;
   if (stage < 1) return ERR_UNSUPPORTED_SIZE;
   a.stage = stage;
-  const size_t lds = (size_t)stage * token_floats * sizeof(float);
+  *lds = (size_t)stage * token_floats * sizeof(float);
+  return 0;
+}
+
+#define LS_LAUNCH(MODE_, grid_, threads_, lds_)                                                                   \
+  do {                                                                                                            \
+    if (dtype == DT_F32) {                                                                                        \
+      if (delta) linear_state_scan_kernel<float, true, MODE_><<<grid_, threads_, lds_, stream>>>(a);              \
+      else linear_state_scan_kernel<float, false, MODE_><<<grid_, threads_, lds_, stream>>>(a);                   \
+    } else {                                                                                                      \
+      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_><<<grid_, threads_, lds_, stream>>>(a);             \
+      else linear_state_scan_kernel<bf16_t, false, MODE_><<<grid_, threads_, lds_, stream>>>(a);                  \
+    }                                                                                                             \
+  } while (0)
+
+extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col, int k_col, int v_col, int removal_col,
+                                    int H, int dk, int dv, float* state, const int* cu_seqlens, const int* slot_ids,
+                                    int lanes, float* out, long out_ld, int max_query_len, const float* head_decay,
+                                    float key_scale, const int* positions, const float* inv_freq, int rotary_dim,
+                                    const float* decay_logits, long logits_ld, const float* decay_bias,
+                                    float decay_floor, float key_eps, hipStream_t stream) {
+  if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_ARGUMENT;
+  ScanArgs a;
+  int code = scan_args(a, u, ld, q_col, k_col, v_col, removal_col, H, dk, dv, state, cu_seqlens, slot_ids, lanes, out,
+                       out_ld, head_decay, key_scale, positions, inv_freq, rotary_dim, decay_logits, logits_ld,
+                       decay_bias, decay_floor, key_eps);
+  if (code) return code;
+  const bool delta = removal_col >= 0;
+  const int threads = max_query_len == 1 ? WAVE : LS_THREADS;
+  size_t lds;
+  int splits;
+  code = scan_shape(a, threads, dv, delta, max_query_len, &lds, &splits);
+  if (code) return code;
   const dim3 grid(lanes, H, splits);
-#define LAUNCH(T_, DELTA_) linear_state_scan_kernel<T_, DELTA_><<<grid, threads, lds, stream>>>(a)
-  if (dtype == DT_F32) { if (delta) LAUNCH(float, true); else LAUNCH(float, false); }
-  else if (dtype == DT_BF16) { if (delta) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
-  else return ERR_BAD_ARGUMENT;
-#undef LAUNCH
+  LS_LAUNCH(LS_WHOLE, grid, threads, lds);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// floats of the two workspaces of the passes over ``chunks`` chunks
+extern "C" long mi_linear_state_local_floats(int chunks, int H, int dk, int dv, int delta) {
+  return (long)chunks * H * (delta ? dv + dk : dv) * dk;
+}
+extern "C" long mi_linear_state_start_floats(int chunks, int H, int dk, int dv) { return (long)chunks * H * dv * dk; }
+
+// The same scan in three passes over the step's chunks (see the top of the file).  ``chunks`` int32 [num_chunks, 4],
+// ``lane_chunks`` int32 [lanes, 2]; ``local`` and ``start``: float32 workspaces of the sizes above.
+extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, int q_col, int k_col, int v_col,
+                                            int removal_col, int H, int dk, int dv, float* state,
+                                            const int* cu_seqlens, const int* slot_ids, int lanes, float* out,
+                                            long out_ld, int chunk_tokens, const float* head_decay, float key_scale,
+                                            const int* positions, const float* inv_freq, int rotary_dim,
+                                            const float* decay_logits, long logits_ld, const float* decay_bias,
+                                            float decay_floor, float key_eps, const int* chunks, const int* lane_chunks,
+                                            int num_chunks, float* local, float* start, hipStream_t stream) {
+  if (dtype != DT_F32 && dtype != DT_BF16) return ERR_BAD_ARGUMENT;
+  if (!chunks || !lane_chunks || num_chunks <= 0 || !local || !start || chunk_tokens <= 0) return ERR_BAD_ARGUMENT;
+  ScanArgs a;
+  int code = scan_args(a, u, ld, q_col, k_col, v_col, removal_col, H, dk, dv, state, cu_seqlens, slot_ids, lanes, out,
+                       out_ld, head_decay, key_scale, positions, inv_freq, rotary_dim, decay_logits, logits_ld,
+                       decay_bias, decay_floor, key_eps);
+  if (code) return code;
+  a.chunks = chunks; a.lane_chunks = lane_chunks; a.local = local; a.start = start;
+  const bool delta = removal_col >= 0;
+  size_t lds;
+  int splits;
+  // local: the chunks' own states (and transitions)
+  code = scan_shape(a, LS_THREADS, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
+  if (code) return code;
+  LS_LAUNCH(LS_LOCAL, dim3(num_chunks, H, splits), LS_THREADS, lds);
+  RETURN_IF_LAUNCH_FAILED();
+  // carry: every chunk's starting state
+  const int carry_splits = (dv + LS_CARRY_COLUMNS - 1) / LS_CARRY_COLUMNS;
+  if (carry_splits > 65535) return ERR_UNSUPPORTED_SIZE;
+  int carry_threads = ((dk + WAVE - 1) / WAVE) * WAVE;
+  if (carry_threads > LS_THREADS) carry_threads = LS_THREADS;
+  const size_t carry_lds = (size_t)LS_CARRY_COLUMNS * dk * sizeof(float);
+  if (delta) linear_state_carry_kernel<true><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
+  else linear_state_carry_kernel<false><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
+  RETURN_IF_LAUNCH_FAILED();
+  // scan: the outputs, and the requests' states behind their last chunks
+  code = scan_shape(a, LS_THREADS, dv, delta, chunk_tokens, &lds, &splits);
+  if (code) return code;
+  LS_LAUNCH(LS_CHUNK, dim3(num_chunks, H, splits), LS_THREADS, lds);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -147,7 +147,11 @@ class Engine:
         self.halves_share: Optional[float] = None
         if decode_graphs and check_device and self.model.graph_safe:
             from .graphs import DecodeGraphs
-            self.graphs = DecodeGraphs(self.model, self.cache, self.device, min(self.max_context, capacity))
+            # the pool bounds a request's length only where some layer keeps every key: a model whose attention
+            # layers all have windows (or that has none) gives passed pages back, and a request outgrows the pool
+            bound = any(group.need.window is None for group in self.cache.groups)
+            self.graphs = DecodeGraphs(self.model, self.cache, self.device,
+                                       min(self.max_context, capacity) if bound else self.max_context)
 
     @property
     def split_from_lanes(self) -> int:

@@ -94,7 +94,7 @@ class DecoderModel:
             self.lm_head = self.embedding
         else:
             head = tensors[f"{spec.lm_head_name}.weight"]
-            if build.dtype == torch.float32:
+            if build.dtype == torch.float32 or spec.hidden_size % 8 != 0:     # rows of no whole 16-byte pieces: see Linear
                 head = head.to(torch.float32)
             self.lm_head = head.contiguous().to(build.device)
         # the copy of the head that the skinny kernel streams fastest, for steps that want few rows

@@ -48,6 +48,12 @@ _SIGNATURES = {
         "mi_linear_state_scan": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
                                  _c_ptr, _c_ptr, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int,
                                  _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_ptr],
+        "mi_linear_state_scan_chunked": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                         _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_long, _c_int, _c_ptr, _c_float, _c_ptr,
+                                         _c_ptr, _c_int, _c_ptr, _c_long, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr,
+                                         _c_int, _c_ptr, _c_ptr, _c_ptr],
+        "mi_linear_state_local_floats": [_c_int, _c_int, _c_int, _c_int, _c_int],
+        "mi_linear_state_start_floats": [_c_int, _c_int, _c_int, _c_int],
         "mi_head_norm_gate": [_c_ptr, _c_long, _c_ptr, _c_int, _c_long, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr,
                               _c_long, _c_int, _c_ptr],
         "mi_tanh_rows": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_int, _c_int, _c_ptr],
@@ -366,7 +372,7 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
                       key_scale: float = 1.0, positions: Optional[torch.Tensor] = None,
                       inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0, removal_col: int = -1,
                       decay_logits: Optional[torch.Tensor] = None, decay_bias: Optional[torch.Tensor] = None,
-                      decay_floor: float = 0.0, key_eps: float = 0.0) -> None:
+                      decay_floor: float = 0.0, key_eps: float = 0.0, chunks=None) -> None:
     """The scan of a mixer whose state is a matrix per head, from and into ``state`` [slots, H, dv, dk] (float32, the
     state of a head transposed), for every lane of the step from its slot; ``out`` float32 [T, H * dv] = S^T q.
 
@@ -376,7 +382,10 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
     Delta rule (``removal_col`` >= 0: the columns of the removal rate's logits; ``decay_logits`` float32 [T, H * dk],
     ``decay_bias`` float32 [H * dk]): w = exp(-decay_floor * sigmoid(logits + bias)), a = sigmoid(removal),
     u = k / sqrt(sum k^2 + key_eps), S <- diag(w) S - (a u)(u^T S) + k v^T.  ``max_query_len``: the longest lane
-    (1 picks small workgroups; 0: not known)."""
+    (1 picks small workgroups; 0: not known).  ``chunks`` (a table of the step's lanes cut into chunks: ``chunks``
+    int32 [n, 4], ``lane_chunks`` int32 [lanes, 2], ``num_chunks``, ``chunk_size``): the scan runs chunk by chunk in
+    three passes (the chunks' own states and transitions side by side, the carry from chunk to chunk, the outputs
+    side by side), the same sums in another order: for long portions."""
     ld = _row_major(u, "u")
     T = u.shape[0]
     H, dk, dv = int(num_heads), int(key_dim), int(value_dim)
@@ -405,6 +414,24 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
         _i32(positions, "positions")
         _need(positions.numel() == T and inv_freq.dtype == torch.float32 and inv_freq.numel() == rotary_dim // 2
               and inv_freq.is_cuda and 0 < rotary_dim <= dk, "linear_state_scan: the rotation does not fit the heads")
+    if chunks is not None:
+        _i32(chunks.chunks, "chunks")
+        _i32(chunks.lane_chunks, "lane_chunks")
+        count = int(chunks.num_chunks)
+        _need(chunks.chunks.numel() >= 4 * count and chunks.lane_chunks.numel() >= 2 * lanes and count > 0,
+              "linear_state_scan: the chunk table does not cover the step")
+        floats = _fn("linear_state", "mi_linear_state_local_floats", _c_long)(count, H, dk, dv, int(delta))
+        local = torch.empty((floats,), dtype=torch.float32, device=u.device)
+        start = torch.empty((_fn("linear_state", "mi_linear_state_start_floats", _c_long)(count, H, dk, dv),),
+                            dtype=torch.float32, device=u.device)
+        _check(_fn("linear_state", "mi_linear_state_scan_chunked")(
+            _p(u), _dt(u), ld, int(q_col), int(k_col), int(v_col), int(removal_col), H, dk, dv, _p(state),
+            _p(cu_seqlens), _p(slot_ids), lanes, _p(out), out.stride(0), int(chunks.chunk_size), _p(head_decay),
+            float(key_scale), _p(positions) if inv_freq is not None else None, _p(inv_freq),
+            int(rotary_dim) if inv_freq is not None else 0, _p(decay_logits), logits_ld, _p(decay_bias),
+            float(decay_floor), float(key_eps), _p(chunks.chunks), _p(chunks.lane_chunks), count, _p(local), _p(start),
+            _stream()), "linear_state_scan_chunked", f"(dk={dk}, dv={dv}, chunks={count})")
+        return
     _check(_fn("linear_state", "mi_linear_state_scan")(
         _p(u), _dt(u), ld, int(q_col), int(k_col), int(v_col), int(removal_col), H, dk, dv, _p(state), _p(cu_seqlens),
         _p(slot_ids), lanes, _p(out), out.stride(0), int(max_query_len), _p(head_decay), float(key_scale),

@@ -33,6 +33,10 @@ class Linear:
         stored = {w.dtype for w in weights}
         keep = torch.float32 if (build.dtype == torch.float32 or stored != {torch.bfloat16}) else torch.bfloat16
         weight = torch.cat([w.to(torch.float32) for w in weights], dim=0)
+        if weight.shape[1] % 8 != 0:
+            # rows that are no whole number of 16-byte pieces in bfloat16: the library's kernels load such pieces;
+            # the product goes through this package's own float32 kernel, which takes any width
+            keep = torch.float32
         rows = weight.shape[0]
         scale = _as_rows(weight_scale, rows)
         if scale is not None:

@@ -17,12 +17,30 @@ from .base import BuildContext, Mixer, part_class, register_part
 from .linear import Linear
 
 
+CHUNK_TOKENS = 128      # lanes longer than this scan in chunks of this many tokens, side by side
+
+
+def scan_chunks(step):
+    """The step's lanes cut into chunks when one of them is long enough for the scan in passes to pay, else None
+    (the scan then walks every lane from end to end, which is what steps of single tokens and short portions want)."""
+    if step.max_query_len <= CHUNK_TOKENS:
+        return None
+    table = step.chunk_tables.get(CHUNK_TOKENS)
+    if table is not None:
+        return table
+    key = ("linear_state_chunks", CHUNK_TOKENS)              # a step that was packed without the table
+    if key not in step.derived:
+        step.derived[key] = ops.SsdChunks(step.lane_lengths, CHUNK_TOKENS, step.token_ids.device)
+    return step.derived[key]
+
+
 @register_part("retention")
 class Retention(Mixer):
     """[q | k | v | g] = one projection of the normed rows; q and k rotated by position, k scaled;
     S <- decay[h] S + k v^T, o = S^T q per head; o / rms(o) per head, times SiLU(g), output projection."""
     graph_safe = True
     kernel_modules = ("common", "linear_state", "gemm")
+    chunk_tokens = CHUNK_TOKENS
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
@@ -67,7 +85,7 @@ class Retention(Mixer):
                               value_dim=spec.value_dim, state=cache.states["state"], cu_seqlens=step.cu_seqlens,
                               slot_ids=step.slot_ids, out=raw, max_query_len=step.max_query_len,
                               head_decay=self.decay, key_scale=spec.key_scale, positions=step.positions,
-                              inv_freq=self.inv_freq, rotary_dim=self.rotary_dim)
+                              inv_freq=self.inv_freq, rotary_dim=self.rotary_dim, chunks=scan_chunks(step))
         gated = torch.empty((x.shape[0], values), dtype=u.dtype, device=x.device)
         ops.head_norm_gate(raw, u[:, 2 * keys + values:], None, spec.num_heads, spec.norm_eps, "silu", gated)
         return self.out_proj(gated)
@@ -81,6 +99,7 @@ class GeneralDelta(Mixer):
     then o / rms(o) per head times the weight ``norm``, times sigmoid(g), output projection."""
     graph_safe = True
     kernel_modules = ("common", "linear_state", "gemm")
+    chunk_tokens = CHUNK_TOKENS
 
     @classmethod
     def expected_tensors(cls, spec, prefix: str, hidden_size: int):
@@ -135,7 +154,8 @@ class GeneralDelta(Mixer):
                               key_dim=spec.head_dim, value_dim=spec.head_dim, state=cache.states["state"],
                               cu_seqlens=step.cu_seqlens, slot_ids=step.slot_ids, out=raw,
                               max_query_len=step.max_query_len, removal_col=4 * inner, decay_logits=logits,
-                              decay_bias=self.decay_bias, decay_floor=spec.decay_floor, key_eps=spec.key_eps)
+                              decay_bias=self.decay_bias, decay_floor=spec.decay_floor, key_eps=spec.key_eps,
+                              chunks=scan_chunks(step))
         gated = torch.empty((x.shape[0], inner), dtype=u.dtype, device=x.device)
         ops.head_norm_gate(raw, u[:, 3 * inner:4 * inner], self.norm_weight, spec.num_heads, spec.norm_eps, "sigmoid",
                            gated)

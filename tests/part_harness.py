@@ -25,7 +25,8 @@ class PartHarness:
                 self.cache.add_request(request)
         self.cache.reserve([(request, x.shape[0]) for request, x in lanes])
         step = build_step_context([Lane(request, [0] * x.shape[0]) for request, x in lanes], self.cache, DEV,
-                                  query_tile=getattr(self.part, "query_tile", 0))
+                                  query_tile=getattr(self.part, "query_tile", 0),
+                                  chunk_sizes=tuple({getattr(self.part, "chunk_tokens", 0)} - {0}))
         x = torch.cat([x for _, x in lanes]).to(self.build.dtype).to(DEV)
         out = self.part.forward(x, step, self.cache.entry((0, "p"))).float().cpu()
         pieces, cursor = [], 0

@@ -258,7 +258,7 @@ def head_norm_gate(raw, gate, weight, num_heads, eps, activation, out):
 
 def linear_state_scan(u, *, q_col, k_col, v_col, num_heads, key_dim, value_dim, state, cu_seqlens, slot_ids, out,
                       max_query_len=0, head_decay=None, key_scale=1.0, positions=None, inv_freq=None, rotary_dim=0,
-                      removal_col=-1, decay_logits=None, decay_bias=None, decay_floor=0.0, key_eps=0.0):
+                      removal_col=-1, decay_logits=None, decay_bias=None, decay_floor=0.0, key_eps=0.0, chunks=None):
     """``state`` [slots, H, value dim, key dim] holds the transposed state of every head."""
     H, K, V = num_heads, key_dim, value_dim
     T = u.shape[0]
