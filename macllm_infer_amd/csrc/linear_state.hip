@@ -69,13 +69,25 @@ struct ScanArgs {
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// sum over the R neighbouring lanes of a column (R a power of two up to 64)
+// sum over the R neighbouring lanes of a column (R a power of two up to 64; a constant R gives constant lane
+// distances, which need no trip through the LDS crossbar)
+template <int R_CONST>
 __device__ __forceinline__ float column_sum(float v, int R) {
-  for (int offset = R >> 1; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+  if (R_CONST > 0) {
+#pragma unroll
+    for (int offset = R_CONST >> 1; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+  } else {
+    for (int offset = R >> 1; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+  }
   return v;
 }
 
-template <typename T, bool DELTA, int MODE>
+__device__ __forceinline__ float dot4(const float4 a, const float* s) {
+  return fmaf(a.w, s[3], fmaf(a.z, s[2], fmaf(a.y, s[1], a.x * s[0])));
+}
+
+// R_CONST: the lanes of a column when the launch knows them at compile time (1 .. 16), 0: a.R
+template <typename T, bool DELTA, int MODE, int R_CONST>
 __global__ void __launch_bounds__(LS_THREADS)
 linear_state_scan_kernel(const ScanArgs a) {
   extern __shared__ __align__(16) float stage_lds[];
@@ -100,11 +112,12 @@ linear_state_scan_kernel(const ScanArgs a) {
   const int wave = tid / WAVE;
   const int lane = tid & (WAVE - 1);
   const int waves = blockDim.x / WAVE;
-  const int R = a.R, per_lane = a.per_lane;
+  const int R = R_CONST > 0 ? R_CONST : a.R;
+  const int per_lane = a.per_lane;                       // a multiple of 4
   const int dk = a.dk, dv = a.dv;
   const int padded = R * per_lane;                       // a vector's length in LDS; channels past dk hold zeros
   const int vectors = DELTA ? 5 : 2;
-  const int token_floats = vectors * padded + a.columns;
+  const int token_floats = vectors * padded + ((a.columns + 3) & ~3);
   const int column_in_group = tid / R;
   const int sub = tid - column_in_group * R;
   const int column = blockIdx.z * a.columns + column_in_group;
@@ -132,56 +145,43 @@ linear_state_scan_kernel(const ScanArgs a) {
   for (int stage_first = first_token; stage_first < end_token; stage_first += a.stage) {
     const int count = min(a.stage, end_token - stage_first);
     __syncthreads();                                       // the stage before is read
-    // ---- lay the stage's vectors in LDS: a wave a token
-    for (int tt = wave; tt < count; tt += waves) {
+    // ---- lay the stage's vectors in LDS: every thread an element (token, channel) at a time, so that the loads
+    // of a whole stage are under way together
+    for (int index = tid; index < count * padded; index += blockDim.x) {
+      const int tt = index / padded;
+      const int channel = index - tt * padded;
       const long token = stage_first + tt;
       const T* row = rows + token * a.ld;
       float* q_lds = stage_lds + tt * token_floats;
-      float* k_lds = q_lds + padded;
-      float sum_squares = 0.f;
-      float position = 0.f;
-      if (!DELTA && a.inv_freq) position = (float)a.positions[token];
-      for (int channel = lane; channel < padded; channel += WAVE) {
-        float qx = 0.f, kx = 0.f;
-        if (channel < dk) {
-          qx = to_float(row[a.q_col + head * dk + channel]);
-          kx = to_float(row[a.k_col + head * dk + channel]);
-          if (!DELTA) {
-            if (a.inv_freq && channel < a.rotary_dim) {
-              const bool low = channel < half;
-              const int pair = low ? channel + half : channel - half;
-              const float angle = position * a.inv_freq[low ? channel : channel - half];
-              const float sine = sinf(angle), cosine = cosf(angle);
-              const float q_pair = to_float(row[a.q_col + head * dk + pair]);
-              const float k_pair = to_float(row[a.k_col + head * dk + pair]);
-              // (x, y) -> (x cos - y sin, y cos + x sin): the low half is x, the high half y
-              qx = low ? qx * cosine - q_pair * sine : qx * cosine + q_pair * sine;
-              kx = low ? kx * cosine - k_pair * sine : kx * cosine + k_pair * sine;
-            }
-            kx *= a.key_scale;
+      float qx = 0.f, kx = 0.f, w = 0.f, removal = 0.f;
+      if (channel < dk) {
+        qx = to_float(row[a.q_col + head * dk + channel]);
+        kx = to_float(row[a.k_col + head * dk + channel]);
+        if (DELTA) {
+          removal = sigmoid_f(to_float(row[a.removal_col + head * dk + channel]));
+          w = expf(-a.decay_floor * sigmoid_f(a.decay_logits[token * a.logits_ld + head * dk + channel] +
+                                              a.decay_bias[head * dk + channel]));
+        } else {
+          if (a.inv_freq && channel < a.rotary_dim) {
+            const bool low = channel < half;
+            const int pair = low ? channel + half : channel - half;
+            const float angle = (float)a.positions[token] * a.inv_freq[low ? channel : channel - half];
+            float sine, cosine;
+            sincosf(angle, &sine, &cosine);
+            const float q_pair = to_float(row[a.q_col + head * dk + pair]);
+            const float k_pair = to_float(row[a.k_col + head * dk + pair]);
+            // (x, y) -> (x cos - y sin, y cos + x sin): the low half is x, the high half y
+            qx = low ? qx * cosine - q_pair * sine : qx * cosine + q_pair * sine;
+            kx = low ? kx * cosine - k_pair * sine : kx * cosine + k_pair * sine;
           }
+          kx *= a.key_scale;
         }
-        q_lds[channel] = qx;
-        k_lds[channel] = kx;
-        sum_squares += kx * kx;
       }
+      q_lds[channel] = qx;
+      q_lds[padded + channel] = kx;
       if (DELTA) {
-        float* w_lds = k_lds + padded;
-        float* u_lds = w_lds + padded;
-        float* au_lds = u_lds + padded;
-        const float length = sqrtf(wave_sum(sum_squares) + a.key_eps);
-        const float* logits = a.decay_logits + token * a.logits_ld + head * dk;
-        for (int channel = lane; channel < padded; channel += WAVE) {
-          float w = 0.f, unit = 0.f, removed = 0.f;
-          if (channel < dk) {
-            unit = k_lds[channel] / length;
-            removed = sigmoid_f(to_float(row[a.removal_col + head * dk + channel])) * unit;
-            w = expf(-a.decay_floor * sigmoid_f(logits[channel] + a.decay_bias[head * dk + channel]));
-          }
-          w_lds[channel] = w;
-          u_lds[channel] = unit;
-          au_lds[channel] = removed;
-        }
+        q_lds[2 * padded + channel] = w;
+        q_lds[4 * padded + channel] = removal;             // times the unit key below
       }
     }
     // the values of this workgroup's columns
@@ -191,6 +191,21 @@ linear_state_scan_kernel(const ScanArgs a) {
       const int value_column = blockIdx.z * a.columns + c;
       stage_lds[tt * token_floats + vectors * padded + c] =
           value_column < dv ? to_float(rows[(long)(stage_first + tt) * a.ld + a.v_col + head * dv + value_column]) : 0.f;
+    }
+    if (DELTA) {
+      __syncthreads();
+      // the unit keys: a wave a token
+      for (int tt = wave; tt < count; tt += waves) {
+        float* k_lds = stage_lds + tt * token_floats + padded;
+        float sum_squares = 0.f;
+        for (int channel = lane; channel < padded; channel += WAVE) sum_squares = fmaf(k_lds[channel], k_lds[channel], sum_squares);
+        const float length = sqrtf(wave_sum(sum_squares) + a.key_eps);
+        for (int channel = lane; channel < padded; channel += WAVE) {
+          const float unit = k_lds[channel] / length;
+          k_lds[2 * padded + channel] = unit;
+          k_lds[3 * padded + channel] *= unit;
+        }
+      }
     }
     __syncthreads();
     // ---- the tokens of the stage in order
@@ -204,27 +219,39 @@ linear_state_scan_kernel(const ScanArgs a) {
           const float* w_lds = k_lds + padded;
           const float* u_lds = w_lds + padded;
           const float* au_lds = u_lds + padded;
-          float along = 0.f;
+          float part[LS_MAX_PER_LANE / 4];
 #pragma unroll
-          for (int e = 0; e < LS_MAX_PER_LANE; ++e)
-            if (e < per_lane) along = fmaf(u_lds[e], s[e], along);
-          along = column_sum(along, R);
+          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+            part[g] = 4 * g < per_lane ? dot4(*reinterpret_cast<const float4*>(u_lds + 4 * g), s + 4 * g) : 0.f;
+          const float along = column_sum<R_CONST>((part[0] + part[1]) + (part[2] + part[3]), R);
 #pragma unroll
-          for (int e = 0; e < LS_MAX_PER_LANE; ++e)
-            if (e < per_lane) {
-              s[e] = fmaf(k_lds[e], value, fmaf(-au_lds[e], along, w_lds[e] * s[e]));
-              if (MODE != LS_LOCAL) result = fmaf(s[e], q_lds[e], result);
+          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+            if (4 * g < per_lane) {
+              const float4 k4 = *reinterpret_cast<const float4*>(k_lds + 4 * g);
+              const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 4 * g);
+              const float4 au4 = *reinterpret_cast<const float4*>(au_lds + 4 * g);
+              s[4 * g + 0] = fmaf(k4.x, value, fmaf(-au4.x, along, w4.x * s[4 * g + 0]));
+              s[4 * g + 1] = fmaf(k4.y, value, fmaf(-au4.y, along, w4.y * s[4 * g + 1]));
+              s[4 * g + 2] = fmaf(k4.z, value, fmaf(-au4.z, along, w4.z * s[4 * g + 2]));
+              s[4 * g + 3] = fmaf(k4.w, value, fmaf(-au4.w, along, w4.w * s[4 * g + 3]));
             }
         } else {
 #pragma unroll
-          for (int e = 0; e < LS_MAX_PER_LANE; ++e)
-            if (e < per_lane) {
-              s[e] = fmaf(k_lds[e], value, decay * s[e]);
-              if (MODE != LS_LOCAL) result = fmaf(s[e], q_lds[e], result);
+          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+            if (4 * g < per_lane) {
+              const float4 k4 = *reinterpret_cast<const float4*>(k_lds + 4 * g);
+              s[4 * g + 0] = fmaf(k4.x, value, decay * s[4 * g + 0]);
+              s[4 * g + 1] = fmaf(k4.y, value, decay * s[4 * g + 1]);
+              s[4 * g + 2] = fmaf(k4.z, value, decay * s[4 * g + 2]);
+              s[4 * g + 3] = fmaf(k4.w, value, decay * s[4 * g + 3]);
             }
         }
         if (MODE != LS_LOCAL) {
-          result = column_sum(result, R);
+          float part[LS_MAX_PER_LANE / 4];
+#pragma unroll
+          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+            part[g] = 4 * g < per_lane ? dot4(*reinterpret_cast<const float4*>(q_lds + 4 * g), s + 4 * g) : 0.f;
+          result = column_sum<R_CONST>((part[0] + part[1]) + (part[2] + part[3]), R);
           if (mine && sub == 0) a.out[(long)(stage_first + tt) * a.out_ld + head * dv + column] = result;
         }
       }
@@ -245,7 +272,7 @@ linear_state_scan_kernel(const ScanArgs a) {
 // One workgroup a (lane, head, run of LS_CARRY_COLUMNS value columns): the columns' states sit in LDS, a thread
 // owns key channels m and computes, for its columns j, s_j[m] <- sum_i P[m, i] s_j[i] + B_j[m] chunk after chunk
 // (P's column i is row dv + i of what the local pass left); every chunk's starting state goes to ``start``.
-#define LS_CARRY_COLUMNS 8
+#define LS_CARRY_COLUMNS 4
 
 template <bool DELTA>
 __global__ void __launch_bounds__(LS_THREADS)
@@ -281,10 +308,18 @@ linear_state_carry_kernel(const ScanArgs a) {
       if (m < dk) {
         if (DELTA) {
           const float* transition = local + (long)dv * dk + m;       // P[m, i] at transition[i * dk]
-          for (int i = 0; i < dk; ++i) {
-            const float p = transition[(long)i * dk];
+          // eight of the transition's elements are asked for before the first is used
+          for (int i0 = 0; i0 < dk; i0 += 8) {
+            float p[8];
 #pragma unroll
-            for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = fmaf(p, carry_lds[c * dk + i], next[c]);
+            for (int j = 0; j < 8; ++j) p[j] = transition[(long)min(i0 + j, dk - 1) * dk];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int i = min(i0 + j, dk - 1);
+              const float weight = i0 + j < dk ? p[j] : 0.f;
+#pragma unroll
+              for (int c = 0; c < LS_CARRY_COLUMNS; ++c) next[c] = fmaf(weight, carry_lds[c * dk + i], next[c]);
+            }
           }
         } else {
 #pragma unroll
@@ -339,7 +374,7 @@ static int scan_args(ScanArgs& a, const void* u, long ld, int q_col, int k_col, 
   int R = 1;
   while (R * LS_MAX_PER_LANE < dk) R *= 2;
   a.R = R;
-  a.per_lane = (dk + R - 1) / R;
+  a.per_lane = (((dk + R - 1) / R + 3) / 4) * 4;           // whole groups of four channels: 16-byte reads from LDS
   return 0;
 }
 
@@ -349,7 +384,7 @@ static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, i
   if (a.columns > total_columns) a.columns = total_columns;
   *splits = (total_columns + a.columns - 1) / a.columns;
   if (*splits > 65535) return ERR_UNSUPPORTED_SIZE;
-  const int token_floats = (delta ? 5 : 2) * a.R * a.per_lane + a.columns;
+  const int token_floats = (delta ? 5 : 2) * a.R * a.per_lane + ((a.columns + 3) & ~3);
   int stage = LS_STAGE_BYTES / (token_floats * (int)sizeof(float));
   if (stage > LS_STAGE_MOST) stage = LS_STAGE_MOST;
   if (longest > 0 && stage > longest) stage = longest;
@@ -359,14 +394,24 @@ static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, i
   return 0;
 }
 
-#define LS_LAUNCH(MODE_, grid_, threads_, lds_)                                                                   \
+#define LS_LAUNCH_R(MODE_, R_, grid_, threads_, lds_)                                                              \
   do {                                                                                                            \
     if (dtype == DT_F32) {                                                                                        \
-      if (delta) linear_state_scan_kernel<float, true, MODE_><<<grid_, threads_, lds_, stream>>>(a);              \
-      else linear_state_scan_kernel<float, false, MODE_><<<grid_, threads_, lds_, stream>>>(a);                   \
+      if (delta) linear_state_scan_kernel<float, true, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);          \
+      else linear_state_scan_kernel<float, false, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);               \
     } else {                                                                                                      \
-      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_><<<grid_, threads_, lds_, stream>>>(a);             \
-      else linear_state_scan_kernel<bf16_t, false, MODE_><<<grid_, threads_, lds_, stream>>>(a);                  \
+      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);         \
+      else linear_state_scan_kernel<bf16_t, false, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);              \
+    }                                                                                                             \
+  } while (0)
+#define LS_LAUNCH(MODE_, grid_, threads_, lds_)                                                                   \
+  do {                                                                                                            \
+    switch (a.R) {                                                                                                \
+      case 1: LS_LAUNCH_R(MODE_, 1, grid_, threads_, lds_); break;                                                \
+      case 2: LS_LAUNCH_R(MODE_, 2, grid_, threads_, lds_); break;                                                \
+      case 4: LS_LAUNCH_R(MODE_, 4, grid_, threads_, lds_); break;                                                \
+      case 8: LS_LAUNCH_R(MODE_, 8, grid_, threads_, lds_); break;                                                \
+      default: LS_LAUNCH_R(MODE_, 0, grid_, threads_, lds_); break;                                               \
     }                                                                                                             \
   } while (0)
 
