@@ -34,6 +34,8 @@
 
 #define LS_MAX_PER_LANE 16          // key channels of a column that one lane keeps
 #define LS_THREADS 256
+#define LS_PASS_THREADS 1024        // a workgroup of the passes over chunks: its many waves hide each other's waits
+#define LS_PASS_LANES 16            // lanes a column there, when the head is wide enough (4 key channels a lane or more)
 #define LS_STAGE_MOST 16            // tokens of a stage
 #define LS_STAGE_BYTES (48 * 1024)
 
@@ -69,13 +71,22 @@ struct ScanArgs {
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// sum over the R neighbouring lanes of a column (R a power of two up to 64; a constant R gives constant lane
-// distances, which need no trip through the LDS crossbar)
+// sum over the R neighbouring lanes of a column (R a power of two up to 64).  A constant R up to 16 stays inside a
+// row of 16 lanes, where the data-parallel primitives exchange lanes without a trip through the LDS crossbar:
+// neighbours in a quad, the quads' other pair, then the mirror image within 8 and within 16 lanes (every lane of
+// a half holds the half's sum by then, so the mirror brings the other half's).
+template <int CONTROL>
+__device__ __forceinline__ float lanes_moved(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CONTROL, 0xf, 0xf, true));
+}
+
 template <int R_CONST>
 __device__ __forceinline__ float column_sum(float v, int R) {
   if (R_CONST > 0) {
-#pragma unroll
-    for (int offset = R_CONST >> 1; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+    if (R_CONST >= 2) v += lanes_moved<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+    if (R_CONST >= 4) v += lanes_moved<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+    if (R_CONST >= 8) v += lanes_moved<0x141>(v);      // row_half_mirror
+    if (R_CONST >= 16) v += lanes_moved<0x140>(v);     // row_mirror
   } else {
     for (int offset = R >> 1; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
   }
@@ -88,7 +99,7 @@ __device__ __forceinline__ float dot4(const float4 a, const float* s) {
 
 // R_CONST: the lanes of a column when the launch knows them at compile time (1 .. 16), 0: a.R
 template <typename T, bool DELTA, int MODE, int R_CONST>
-__global__ void __launch_bounds__(LS_THREADS)
+__global__ void __launch_bounds__(MODE == LS_WHOLE ? LS_THREADS : LS_PASS_THREADS)
 linear_state_scan_kernel(const ScanArgs a) {
   extern __shared__ __align__(16) float stage_lds[];
   const int head = blockIdx.y;
@@ -308,13 +319,13 @@ linear_state_carry_kernel(const ScanArgs a) {
       if (m < dk) {
         if (DELTA) {
           const float* transition = local + (long)dv * dk + m;       // P[m, i] at transition[i * dk]
-          // eight of the transition's elements are asked for before the first is used
-          for (int i0 = 0; i0 < dk; i0 += 8) {
-            float p[8];
+          // 32 of the transition's elements are asked for before the first is used
+          for (int i0 = 0; i0 < dk; i0 += 32) {
+            float p[32];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) p[j] = transition[(long)min(i0 + j, dk - 1) * dk];
+            for (int j = 0; j < 32; ++j) p[j] = transition[(long)min(i0 + j, dk - 1) * dk];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 32; ++j) {
               const int i = min(i0 + j, dk - 1);
               const float weight = i0 + j < dk ? p[j] : 0.f;
 #pragma unroll
@@ -411,6 +422,7 @@ static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, i
       case 2: LS_LAUNCH_R(MODE_, 2, grid_, threads_, lds_); break;                                                \
       case 4: LS_LAUNCH_R(MODE_, 4, grid_, threads_, lds_); break;                                                \
       case 8: LS_LAUNCH_R(MODE_, 8, grid_, threads_, lds_); break;                                                \
+      case 16: LS_LAUNCH_R(MODE_, 16, grid_, threads_, lds_); break;                                              \
       default: LS_LAUNCH_R(MODE_, 0, grid_, threads_, lds_); break;                                               \
     }                                                                                                             \
   } while (0)
@@ -466,10 +478,22 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
   const bool delta = removal_col >= 0;
   size_t lds;
   int splits;
+  // the passes spread a column over more lanes than the walk from end to end: up to LS_PASS_LANES, four key
+  // channels a lane or more, so that a token is a short chain of sums and a workgroup of LS_PASS_THREADS threads
+  // still takes 64 columns with one copy of the stage's vectors
+  {
+    int R = 1;
+    while (R * 4 < dk && R < LS_PASS_LANES) R *= 2;
+    while (R * LS_MAX_PER_LANE < dk) R *= 2;
+    a.R = R;
+    a.per_lane = (((dk + R - 1) / R + 3) / 4) * 4;
+  }
   // local: the chunks' own states (and transitions)
-  code = scan_shape(a, LS_THREADS, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
   if (code) return code;
-  LS_LAUNCH(LS_LOCAL, dim3(num_chunks, H, splits), LS_THREADS, lds);
+  int threads = ((a.columns * a.R + WAVE - 1) / WAVE) * WAVE;          // no more waves than the columns fill
+  if (threads < LS_THREADS) threads = LS_THREADS;
+  LS_LAUNCH(LS_LOCAL, dim3(num_chunks, H, splits), threads, lds);
   RETURN_IF_LAUNCH_FAILED();
   // carry: every chunk's starting state
   const int carry_splits = (dv + LS_CARRY_COLUMNS - 1) / LS_CARRY_COLUMNS;
@@ -481,9 +505,11 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
   else linear_state_carry_kernel<false><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
   RETURN_IF_LAUNCH_FAILED();
   // scan: the outputs, and the requests' states behind their last chunks
-  code = scan_shape(a, LS_THREADS, dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS, dv, delta, chunk_tokens, &lds, &splits);
   if (code) return code;
-  LS_LAUNCH(LS_CHUNK, dim3(num_chunks, H, splits), LS_THREADS, lds);
+  threads = ((a.columns * a.R + WAVE - 1) / WAVE) * WAVE;
+  if (threads < LS_THREADS) threads = LS_THREADS;
+  LS_LAUNCH(LS_CHUNK, dim3(num_chunks, H, splits), threads, lds);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
