@@ -983,13 +983,16 @@ extern "C" int mi_decode_attention_static(const void* q, long q_ld, int T, int H
 #define PREFILL_WAVES 8
 #define PREFILL_FILL_BLOCKS 512   // two workgroups for each of the 256 compute units
 
-template <int DH, int NSET>
+// EXTRAS: the scores lose log_bias[head] = (r1, r2) -> r1 * ln(1 + r2 * distance), and the softmax's denominator
+// holds one more term exp(sinks[head]) (either pointer may be null).
+template <int DH, int NSET, bool EXTRAS = false>
 __global__ void __launch_bounds__(PREFILL_WAVES * WAVE)
 prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hkv, const bf16_t* __restrict__ k_base,
                          const bf16_t* __restrict__ v_base, long page_stride, int page_size,
                          const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale,
-                         int window, bf16_t* __restrict__ out, long out_ld) {
+                         int window, bf16_t* __restrict__ out, long out_ld,
+                         const float* __restrict__ log_bias = nullptr, const float* __restrict__ sinks = nullptr) {
   constexpr int ITEMS = 2 + 4 * (DH / 16);                    // m, l and the accumulator of one set
   __shared__ float part[PREFILL_WAVES][ITEMS][WAVE];
   __shared__ int wave_pages[PREFILL_WAVES][WAVE];
@@ -1037,6 +1040,16 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
   }
   AttnAccumulator<DH, NSET> acc;
   acc.clear();
+  AttnLogBias<NSET> bias;
+  if (EXTRAS) {
+    bias.on = log_bias != nullptr;
+#pragma unroll
+    for (int s = 0; s < NSET; ++s) {
+      const int head = min(head0 + s, Hq - 1);
+      bias.r1[s] = log_bias ? log_bias[2 * head] : 0.f;
+      bias.r2[s] = log_bias ? log_bias[2 * head + 1] : 0.f;
+    }
+  }
   AttnCache cache;
   cache.k_base = k_base;
   cache.v_base = v_base;
@@ -1059,8 +1072,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
     cache.pages = wave_pages[wave];
     cache.base_page = first_page;
-    attend_keys<DH, NSET, PREFILL_STEPS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache,
-                                         full_tile ? first_position : -1, last_position);
+    attend_keys<DH, NSET, PREFILL_STEPS, false, EXTRAS>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache,
+                                                        full_tile ? first_position : -1, last_position, bias);
     part_lo = part_hi;
   }
 
@@ -1079,6 +1092,9 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     float m = -INFINITY;
 #pragma unroll
     for (int w = 0; w < PREFILL_WAVES; ++w) m = fmaxf(m, part[w][0][lane]);
+    // the sink, in the scores' units of log2: it may be the largest term
+    const float sink = (EXTRAS && sinks) ? sinks[min(head0 + s, Hq - 1)] * 1.4426950408889634f : -INFINITY;
+    m = fmaxf(m, sink);
     float factor[PREFILL_WAVES];
     float l = 0.f;
 #pragma unroll
@@ -1089,6 +1105,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int Hq, int Hk
     }
     l += __shfl_xor(l, 16, WAVE);
     l += __shfl_xor(l, 32, WAVE);
+    if (EXTRAS && sinks) l += __builtin_amdgcn_exp2f(sink - m);       // once for the column: no key, no value
     if (col_pos[s] < 0) continue;
     const float inverse = 1.f / l;
     bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * DH;
@@ -1113,7 +1130,7 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
                                     const void* v_base, long page_stride, int page_size, const int* block_tables,
                                     int max_pages, const int* tiles, int n_tiles, const int* cu_seqlens,
                                     const int* start_pos, float scale, int window, int max_seq_len, void* out,
-                                    long out_ld, hipStream_t stream) {
+                                    long out_ld, const float* log_bias, const float* sinks, hipStream_t stream) {
   if (n_tiles <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || page_size <= 0 || max_pages <= 0)
     return ERR_BAD_ARGUMENT;
   const int G = Hq / Hkv;
@@ -1132,11 +1149,18 @@ extern "C" int mi_prefill_attention(const void* q, long q_ld, int Hq, int Hkv, i
   const int nset = (G + passes - 1) / passes;
   if (n_tiles > (1 << 28)) return ERR_UNSUPPORTED_SIZE;
   const dim3 grid(4 * n_tiles, Hkv, passes);
+  const bool extras = log_bias != nullptr || sinks != nullptr;
 #define PREFILL_CASE(DH_, NSET_)                                                                              \
-  if (dh == DH_ && nset == NSET_)                                                                             \
-    prefill_attention_kernel<DH_, NSET_><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                                           \
-        (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
-        block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld);
+  if (dh == DH_ && nset == NSET_) {                                                                           \
+    if (extras)                                                                                               \
+      prefill_attention_kernel<DH_, NSET_, true><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                  \
+          (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
+          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, log_bias, sinks); \
+    else                                                                                                      \
+      prefill_attention_kernel<DH_, NSET_><<<grid, PREFILL_WAVES * WAVE, 0, stream>>>(                        \
+          (const bf16_t*)q, q_ld, Hq, Hkv, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, \
+          block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld);         \
+  }
   PREFILL_CASE(64, 1) PREFILL_CASE(64, 2) PREFILL_CASE(64, 3) PREFILL_CASE(64, 4)
   PREFILL_CASE(128, 1) PREFILL_CASE(128, 2) PREFILL_CASE(128, 3) PREFILL_CASE(128, 4)
 #undef PREFILL_CASE

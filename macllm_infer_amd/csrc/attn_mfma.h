@@ -98,15 +98,25 @@ __device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS>& f, int k00, 
   }
 }
 
+// A bias on the scores that grows with the logarithm of the distance: score -= r1 * ln(1 + r2 * (position - key)),
+// one (r1, r2) for each set of columns (a query head).  In units of log2, where the scores live, that is
+// r1 * log2(1 + r2 * distance).  ``on`` false: no bias (the kernels that know none pass the default).
+template <int NSET>
+struct AttnLogBias {
+  bool on = false;
+  float r1[NSET];
+  float r2[NSET];
+};
+
 // Scores, softmax step and values of the loaded steps, per set of columns.
 // MASKED = false: the caller vouches that every key of the round is visible to every column
 // and lies inside the run (steps away from the diagonal, the window's edge and the run's end):
 // no masks are computed.
-template <int DH, int NSET, int STEPS, bool MASKED = true>
+template <int DH, int NSET, int STEPS, bool MASKED = true, bool BIASED = false>
 __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, AttnFragments<DH, STEPS>& f,
                                              const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                              const int (&col_pos)[NSET], int window, float scale, int k00,
-                                             int key_hi) {
+                                             int key_hi, const AttnLogBias<NSET>& bias = AttnLogBias<NSET>()) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int q = lane / 16;
   const int last_key = key_hi - 1;
@@ -143,6 +153,17 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
           score[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[st][t][kk], q_frag[s][kk], score[t], 0, 0, 0);
       }
       // scores in units of log2: s * scale * log2(e), so that the exponentials are bare v_exp
+      if (BIASED) {
+        // the biased scores, already in units of log2 (the scale below is then one); a key past the column's
+        // position gives a logarithm of anything, which the mask replaces
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float distance = (float)(col_pos[s] - (k0 + 16 * t + 4 * q + i));
+            score[t][i] = fmaf(score[t][i], scale_log2, -bias.r1[s] * __log2f(fmaf(bias.r2[s], fmaxf(distance, 0.f), 1.f)));
+          }
+      }
       if (MASKED) {
         // visible keys of the column: first_visible .. min(position, last_key); relative to the step
         // they are lo .. lo + span, so one unsigned compare per score decides (an empty range gets
@@ -165,7 +186,7 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
                              fmaxf(fmaxf(score[1][0], score[1][1]), fmaxf(score[1][2], score[1][3])));
       step_max = fmaxf(step_max, __shfl_xor(step_max, 16, WAVE));
       step_max = fmaxf(step_max, __shfl_xor(step_max, 32, WAVE));
-      step_max *= scale_log2;                                        // scale > 0: the maximum stays the maximum
+      if (!BIASED) step_max *= scale_log2;                           // scale > 0: the maximum stays the maximum
       const float m_new = fmaxf(acc.m[s], step_max);
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;       // nothing visible yet
       const float correction = __builtin_amdgcn_exp2f(acc.m[s] - m_safe);
@@ -176,7 +197,7 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float p = __builtin_amdgcn_exp2f(fmaf(score[t][i], scale_log2, -m_safe));
+          const float p = __builtin_amdgcn_exp2f(BIASED ? score[t][i] - m_safe : fmaf(score[t][i], scale_log2, -m_safe));
           sum += p;
           p_frag[4 * t + i] = (bf16_t)p;
         }
@@ -200,11 +221,12 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
 // with long runs; a caller whose run is one round of STEPS steps gains nothing from it.
 // min_pos / max_pos: the smallest and largest position among the columns of the wave, when all
 // of them hold queries and the caller knows (the same value in every lane), else -1.
-template <int DH, int NSET, int STEPS, bool PIPELINED = false>
+template <int DH, int NSET, int STEPS, bool PIPELINED = false, bool BIASED = false>
 __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
                                             const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                             const int (&col_pos)[NSET], int window, float scale, int key_lo,
-                                            int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1) {
+                                            int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1,
+                                            const AttnLogBias<NSET>& bias = AttnLogBias<NSET>()) {
   const int last_key = key_hi - 1;
   constexpr int ROUND = 32 * STEPS;
   if (PIPELINED) {
@@ -227,12 +249,12 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
     for (int k00 = key_lo; k00 < open_hi; k00 += ROUND) {
       AttnFragments<DH, STEPS> f;
       attn_load<DH, STEPS>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, false>(acc, f, q_frag, col_pos, window, scale, k00, key_hi);
+      attn_compute<DH, NSET, STEPS, false, BIASED>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
     }
     for (int k00 = open_hi; k00 < key_hi; k00 += ROUND) {
       AttnFragments<DH, STEPS> f;
       attn_load<DH, STEPS>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, true>(acc, f, q_frag, col_pos, window, scale, k00, key_hi);
+      attn_compute<DH, NSET, STEPS, true, BIASED>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
     }
   }
 }

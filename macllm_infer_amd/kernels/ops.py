@@ -67,7 +67,7 @@ _SIGNATURES = {
         "mi_paged_attention_workspace": [_c_int, _c_int, _c_int, _c_int],
         "mi_prefill_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr,
                                  _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_ptr, _c_long,
-                                 _c_ptr],
+                                 _c_ptr, _c_ptr, _c_ptr],
         "mi_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                 _c_ptr, _c_long, _c_ptr],
@@ -441,6 +441,9 @@ def linear_state_scan(u: torch.Tensor, *, q_col: int, k_col: int, v_col: int, nu
 
 
 # --------------------------------------------------------------------------- matrix products
+SKINNY_ROWS = 16          # steps of up to this many rows take the skinny kernel in ``linear``
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], keep_float32: bool = False) -> torch.Tensor:
     """x [M, K] . weight[N, K]^T (+ bias float32 [N]) -> [M, N] in x's dtype, or, with
     ``keep_float32`` and no bias, in float32 whatever the operands are (the library writes its
@@ -463,6 +466,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], 
                "gemm_f32", f"(M={M}, N={N}, K={K})")
         return out if x.dtype == torch.float32 or keep_float32 else out.to(x.dtype)
     _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "linear: operands must share a dtype")
+    M, K = x.shape
+    if (M <= SKINNY_ROWS and x.is_cuda and K % 32 == 0 and weight.is_contiguous() and x.stride(1) == 1
+            and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and fused_gemm_supported(False, M, K)):
+        # a step of a few rows waits for the weights: the skinny kernel streams them once, bias and rounding in
+        # its epilogue (the library takes 8 us for such a product where this takes 5)
+        out = torch.empty((M, weight.shape[0]), dtype=torch.float32 if keep_float32 else torch.bfloat16, device=x.device)
+        fused_gemm(weight, bias, out, x=x)
+        return out
     if keep_float32:
         _need(bias is None, "linear: float32 results of bfloat16 operands come without a bias")
         return torch.mm(x, weight.t(), out_dtype=torch.float32)
@@ -597,7 +608,8 @@ def prefill_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_d
 def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, block_tables: torch.Tensor, query_tiles: torch.Tensor,
                       cu_seqlens: torch.Tensor, start_pos: torch.Tensor, scale: float, window: Optional[int],
-                      out: torch.Tensor, max_seq_len: int = 0) -> None:
+                      out: torch.Tensor, max_seq_len: int = 0, log_bias: Optional[torch.Tensor] = None,
+                      sinks: Optional[torch.Tensor] = None) -> None:
     """``paged_attention`` on the matrix cores for bfloat16 (flash-style, online softmax in
     float32).  ``query_tiles`` [tiles, 2]: (lane, first token row) of runs of up to 64 tokens of
     one lane; the keys and values of the step's own tokens must be in the cache already.
@@ -618,11 +630,17 @@ def prefill_attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         _i32(tensor, name)
     _need(block_tables.dim() == 2 and query_tiles.dim() == 2 and query_tiles.shape[1] == 2
           and cu_seqlens.numel() == start_pos.numel() + 1, "prefill_attention: metadata shapes do not match")
+    # the same two terms as ``paged_attention``'s: a bias by the logarithm of the distance, a sink in the denominator
+    _need(log_bias is None or (log_bias.dtype == torch.float32 and log_bias.shape == (num_heads, 2)
+                               and log_bias.is_contiguous() and log_bias.is_cuda),
+          "prefill_attention: log_bias must be float32 [Hq, 2] on the GPU")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == num_heads and sinks.is_contiguous()
+                            and sinks.is_cuda), "prefill_attention: sinks must be float32 [Hq] on the GPU")
     _check(_fn("attention", "mi_prefill_attention")(
         _p(q), q_ld, num_heads, num_kv_heads, head_dim, _p(k_cache), _p(v_cache), page_stride, page_size,
         _p(block_tables), block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens),
-        _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, _stream()),
-        "prefill_attention")
+        _p(start_pos), float(scale), int(window or 0), int(max_seq_len or 0), _p(out), out_ld, _p(log_bias),
+        _p(sinks), _stream()), "prefill_attention")
 
 
 def decode_attention_supported(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> bool:

@@ -115,6 +115,17 @@ class Attention(Mixer):
             tiles = {}
             if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
                 tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
+            if (tiles and slopes is None and spec.value_width == spec.head_dim and step.query_tile == self.query_tile
+                    and ops.prefill_attention_supported(qkv.dtype, *geometry, cache.k_cache.shape[2])
+                    and qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 and attended.stride(0) % 4 == 0
+                    and attended.data_ptr() % 8 == 0):
+                # prompt portions in bfloat16 with heads of 64 or 128: the matrix-core kernel knows the logarithmic
+                # bias and the sink
+                ops.prefill_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
+                                      step.query_tiles, step.cu_seqlens, step.start_pos, spec.scale, spec.window,
+                                      attended, step.max_seq_len, log_bias=self.position.score_log_bias,
+                                      sinks=self.sink)
+                return
             ops.paged_attention(qkv, *geometry, cache.k_cache, cache.v_cache, step.block_tables[cache.group],
                                 step.lane_of_token, step.positions, spec.scale, spec.window, attended,
                                 step.max_seq_len, slopes, log_bias=self.position.score_log_bias, sinks=self.sink,
