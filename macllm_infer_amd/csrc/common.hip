@@ -385,7 +385,7 @@ extern "C" int mi_add_bias_round(const float* sums, const float* bias, void* out
 // or, for wider rows, in LDS.  The sum of squares is added up in an order that d alone fixes.
 #define SCALED_MAX_ROUNDS 8
 template <typename TD, typename TO, bool IN_LDS>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 add_scaled_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ scale,
                           const float* __restrict__ weight, float eps, TO* __restrict__ out,
                           const int* __restrict__ rows, int d) {
@@ -398,7 +398,7 @@ add_scaled_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, c
   float kept[SCALED_MAX_ROUNDS];
   float sum_squares = 0.f;
   if (IN_LDS) {
-    for (int i = threadIdx.x; i < d; i += 256) {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
       const float v = fmaf(scale[i], to_float(dr[i]), hr[i]);
       if (!rows) hr[i] = v;
       wide_row[i] = v;
@@ -407,7 +407,7 @@ add_scaled_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, c
   } else {
 #pragma unroll
     for (int r = 0; r < SCALED_MAX_ROUNDS; ++r) {
-      const int i = (int)threadIdx.x + r * 256;
+      const int i = (int)threadIdx.x + r * (int)blockDim.x;
       const int at = min(i, d - 1);
       const float v = fmaf(scale[at], to_float(dr[at]), hr[at]);
       kept[r] = v;
@@ -422,11 +422,11 @@ add_scaled_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, c
   const float denominator = sqrtf(total / (float)d + eps);
   TO* o = out + out_row * d;
   if (IN_LDS) {
-    for (int i = threadIdx.x; i < d; i += 256) o[i] = from_float<TO>(wide_row[i] / denominator * weight[i]);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_float<TO>(wide_row[i] / denominator * weight[i]);
   } else {
 #pragma unroll
     for (int r = 0; r < SCALED_MAX_ROUNDS; ++r) {
-      const int i = (int)threadIdx.x + r * 256;
+      const int i = (int)threadIdx.x + r * (int)blockDim.x;
       if (i < d) o[i] = from_float<TO>(kept[r] / denominator * weight[i]);
     }
   }
@@ -436,16 +436,18 @@ extern "C" int mi_add_scaled_rmsnorm(float* h, const void* delta, int delta_dtyp
                                      const float* weight, float eps, void* out, int out_dtype, const int* rows,
                                      int n_rows, int d, hipStream_t stream) {
   if (!h || !delta || !scale || !weight || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
-  const bool in_lds = d > 256 * SCALED_MAX_ROUNDS;
+  // a narrow row takes 256 threads; a wide one 1,024, so that a step of few rows still has waves to hide its waits
+  const int threads = d > 2048 ? 1024 : 256;
+  const bool in_lds = d > threads * SCALED_MAX_ROUNDS;
   if (in_lds && (size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   const size_t lds = in_lds ? (size_t)d * sizeof(float) : 0;
 #define LAUNCH(TD, TO)                                                                                              \
   do {                                                                                                              \
     if (in_lds)                                                                                                     \
-      add_scaled_rmsnorm_kernel<TD, TO, true><<<n_rows, 256, lds, stream>>>(h, (const TD*)delta, scale, weight, eps, \
+      add_scaled_rmsnorm_kernel<TD, TO, true><<<n_rows, threads, lds, stream>>>(h, (const TD*)delta, scale, weight, eps, \
                                                                             (TO*)out, rows, d);                     \
     else                                                                                                            \
-      add_scaled_rmsnorm_kernel<TD, TO, false><<<n_rows, 256, 0, stream>>>(h, (const TD*)delta, scale, weight, eps,  \
+      add_scaled_rmsnorm_kernel<TD, TO, false><<<n_rows, threads, 0, stream>>>(h, (const TD*)delta, scale, weight, eps,  \
                                                                            (TO*)out, rows, d);                      \
   } while (0)
   if (delta_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
@@ -463,13 +465,13 @@ extern "C" int mi_add_scaled_rmsnorm(float* h, const void* delta, int delta_dtyp
 // row of x^2 + eps): the three sums of squares of a token's row (z^2, z^4, z^6) in float32, one pass; the row is
 // read a second time (it is in cache) for the result.  One workgroup a row.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 polynorm_kernel(const T* __restrict__ z, long ld, const float* __restrict__ coefficients, float eps,
                 T* __restrict__ out, long out_ld, int I) {
   __shared__ float scratch[16];
   const T* zr = z + (long)blockIdx.x * ld;
   float first = 0.f, second = 0.f, third = 0.f;
-  for (int i = threadIdx.x; i < I; i += 256) {
+  for (int i = threadIdx.x; i < I; i += blockDim.x) {
     const float x = to_float(zr[i]);
     const float x2 = x * x;
     first += x2;
@@ -484,7 +486,7 @@ polynorm_kernel(const T* __restrict__ z, long ld, const float* __restrict__ coef
   const float c = coefficients[2] / sqrtf(mean3 + eps);
   const float e = coefficients[3];
   T* o = out + (long)blockIdx.x * out_ld;
-  for (int i = threadIdx.x; i < I; i += 256) {
+  for (int i = threadIdx.x; i < I; i += blockDim.x) {
     const float x = to_float(zr[i]);
     o[i] = from_float<T>(fmaf(x, fmaf(x, fmaf(x, c, b), a), e));
   }
@@ -493,10 +495,11 @@ polynorm_kernel(const T* __restrict__ z, long ld, const float* __restrict__ coef
 extern "C" int mi_polynorm(const void* z, int dtype, long ld, const float* coefficients, float eps, void* out,
                            long out_ld, int T, int I, hipStream_t stream) {
   if (!z || !coefficients || !out || T <= 0 || I <= 0 || ld < I || out_ld < I) return ERR_BAD_ARGUMENT;
+  const int threads = I > 2048 ? 1024 : 256;
   if (dtype == DT_F32)
-    polynorm_kernel<float><<<T, 256, 0, stream>>>((const float*)z, ld, coefficients, eps, (float*)out, out_ld, I);
+    polynorm_kernel<float><<<T, threads, 0, stream>>>((const float*)z, ld, coefficients, eps, (float*)out, out_ld, I);
   else if (dtype == DT_BF16)
-    polynorm_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)z, ld, coefficients, eps, (bf16_t*)out, out_ld, I);
+    polynorm_kernel<bf16_t><<<T, threads, 0, stream>>>((const bf16_t*)z, ld, coefficients, eps, (bf16_t*)out, out_ld, I);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();
