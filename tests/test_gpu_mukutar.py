@@ -259,12 +259,14 @@ def test_the_generalized_delta_rule_alone(dtype, H, D, rank):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_the_polynorm_feed_forward_the_offset_norm_and_a_scaled_branch_alone(dtype):
+@pytest.mark.parametrize("hidden, inner, T", [(56, 136, 37), (2560, 4104, 9), (8200, 2056, 3)])
+def test_the_polynorm_feed_forward_the_offset_norm_and_a_scaled_branch_alone(dtype, hidden, inner, T):
+    """Narrow rows, rows wide enough for the kernels' large workgroups, and rows that no longer fit a thread's
+    registers."""
     from macllm_infer_amd.config import PolyNormFFNSpec, RmsNormSpec
     from macllm_infer_amd.kernels import build
     from macllm_infer_amd.parts import BuildContext, part_class
     from macllm_infer_amd.parts.base import Residual, ScaledBranch
-    hidden, inner, T = 56, 136, 37
     context = BuildContext(hidden_size=hidden, dtype=dtype, device=torch.device(DEV), max_context=64)
     build.ensure_modules(("common", "gemm"))
     tensors = rounded({"p.up.weight": rand(inner, hidden, seed=1, scale=hidden ** -0.5),
