@@ -97,10 +97,13 @@ __device__ __forceinline__ float dot4(const float4 a, const float* s) {
   return fmaf(a.w, s[3], fmaf(a.z, s[2], fmaf(a.y, s[1], a.x * s[0])));
 }
 
-// R_CONST: the lanes of a column when the launch knows them at compile time (1 .. 16), 0: a.R
-template <typename T, bool DELTA, int MODE, int R_CONST>
+// R_CONST: the lanes of a column when the launch knows them at compile time (1 .. 16), 0: a.R.
+// PL: key channels a lane; a lane keeps 16 / PL neighbouring columns (their states in 16 registers), so that the
+// token's vectors come out of LDS once for all of them.  PL = 16: one column, a.per_lane (<= 16) channels of it.
+template <typename T, bool DELTA, int MODE, int R_CONST, int PL>
 __global__ void __launch_bounds__(MODE == LS_WHOLE ? LS_THREADS : LS_PASS_THREADS)
 linear_state_scan_kernel(const ScanArgs a) {
+  constexpr int CPL = LS_MAX_PER_LANE / PL;              // columns a lane
   extern __shared__ __align__(16) float stage_lds[];
   const int head = blockIdx.y;
   int lane_of_step, first_token, end_token;
@@ -124,31 +127,37 @@ linear_state_scan_kernel(const ScanArgs a) {
   const int lane = tid & (WAVE - 1);
   const int waves = blockDim.x / WAVE;
   const int R = R_CONST > 0 ? R_CONST : a.R;
-  const int per_lane = a.per_lane;                       // a multiple of 4
+  const int per_lane = PL < LS_MAX_PER_LANE ? PL : a.per_lane;   // a multiple of 4
   const int dk = a.dk, dv = a.dv;
   const int padded = R * per_lane;                       // a vector's length in LDS; channels past dk hold zeros
   const int vectors = DELTA ? 5 : 2;
   const int token_floats = vectors * padded + ((a.columns + 3) & ~3);
-  const int column_in_group = tid / R;
-  const int sub = tid - column_in_group * R;
-  const int column = blockIdx.z * a.columns + column_in_group;
+  const int group = tid / R;                             // the lanes of one run of CPL columns
+  const int sub = tid - group * R;
+  const int column_in_group = group * CPL;               // the first of this lane's columns among the workgroup's
+  const int column0 = blockIdx.z * a.columns + column_in_group;
   // the local pass of the delta rule carries dk more columns: the transition's, which start as the unit vectors
   const int total_columns = (MODE == LS_LOCAL && DELTA) ? dv + dk : dv;
-  const bool mine = column_in_group < a.columns && column < total_columns;
+  const bool in_group = column_in_group < a.columns;
   const int channel0 = sub * per_lane;
   const T* rows = (const T*)a.u;
 
-  // the column's share of the state
-  float s[LS_MAX_PER_LANE];
-  float* state_column = a.state + (((long)a.slot_ids[lane_of_step] * a.H + head) * dv + (mine && column < dv ? column : 0)) * dk;
-  const float* from = state_column;
-  if (MODE == LS_CHUNK) from = a.start + (((long)blockIdx.x * a.H + head) * dv + (mine ? column : 0)) * dk;
+  // the columns' share of the state
+  float s[CPL][PL];
+  const long state_head = ((long)a.slot_ids[lane_of_step] * a.H + head) * dv;
 #pragma unroll
-  for (int e = 0; e < LS_MAX_PER_LANE; ++e) {
-    const int channel = channel0 + e;
-    const bool held = mine && e < per_lane && channel < dk;
-    if (MODE == LS_LOCAL) s[e] = (held && channel == column - dv) ? 1.f : 0.f;
-    else s[e] = held ? from[channel] : 0.f;
+  for (int c = 0; c < CPL; ++c) {
+    const int column = column0 + c;
+    const bool mine = in_group && column_in_group + c < a.columns && column < total_columns;
+    const float* from = a.state + (state_head + (mine && column < dv ? column : 0)) * dk;
+    if (MODE == LS_CHUNK) from = a.start + (((long)blockIdx.x * a.H + head) * dv + (mine ? column : 0)) * dk;
+#pragma unroll
+    for (int e = 0; e < PL; ++e) {
+      const int channel = channel0 + e;
+      const bool held = mine && e < per_lane && channel < dk;
+      if (MODE == LS_LOCAL) s[c][e] = (held && channel == column - dv) ? 1.f : 0.f;
+      else s[c][e] = held ? from[channel] : 0.f;
+    }
   }
   const float decay = DELTA ? 0.f : a.head_decay[head];
   const int half = a.rotary_dim / 2;
@@ -220,61 +229,99 @@ linear_state_scan_kernel(const ScanArgs a) {
     }
     __syncthreads();
     // ---- the tokens of the stage in order
-    if (column_in_group < a.columns) {
+    if (in_group) {
       for (int tt = 0; tt < count; ++tt) {
         const float* q_lds = stage_lds + tt * token_floats + channel0;
         const float* k_lds = q_lds + padded;
-        const float value = stage_lds[tt * token_floats + vectors * padded + column_in_group];
-        float result = 0.f;
+        const float* values = stage_lds + tt * token_floats + vectors * padded + column_in_group;
+        float value[CPL];
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) value[c] = values[CPL > 1 ? min(c, a.columns - 1 - column_in_group) : 0];
         if (DELTA) {
           const float* w_lds = k_lds + padded;
           const float* u_lds = w_lds + padded;
           const float* au_lds = u_lds + padded;
-          float part[LS_MAX_PER_LANE / 4];
+          float along[CPL];
 #pragma unroll
-          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
-            part[g] = 4 * g < per_lane ? dot4(*reinterpret_cast<const float4*>(u_lds + 4 * g), s + 4 * g) : 0.f;
-          const float along = column_sum<R_CONST>((part[0] + part[1]) + (part[2] + part[3]), R);
+          for (int c = 0; c < CPL; ++c) along[c] = 0.f;
+          float part[CPL][PL / 4];
 #pragma unroll
-          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+          for (int g = 0; g < PL / 4; ++g) {
+            const bool live = 4 * g < per_lane;
+            const float4 u4 = live ? *reinterpret_cast<const float4*>(u_lds + 4 * g) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) part[c][g] = dot4(u4, s[c] + 4 * g);
+          }
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) {
+            float sum = part[c][0];
+#pragma unroll
+            for (int g = 1; g < PL / 4; ++g) sum += part[c][g];
+            along[c] = column_sum<R_CONST>(sum, R);
+          }
+#pragma unroll
+          for (int g = 0; g < PL / 4; ++g)
             if (4 * g < per_lane) {
               const float4 k4 = *reinterpret_cast<const float4*>(k_lds + 4 * g);
               const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 4 * g);
               const float4 au4 = *reinterpret_cast<const float4*>(au_lds + 4 * g);
-              s[4 * g + 0] = fmaf(k4.x, value, fmaf(-au4.x, along, w4.x * s[4 * g + 0]));
-              s[4 * g + 1] = fmaf(k4.y, value, fmaf(-au4.y, along, w4.y * s[4 * g + 1]));
-              s[4 * g + 2] = fmaf(k4.z, value, fmaf(-au4.z, along, w4.z * s[4 * g + 2]));
-              s[4 * g + 3] = fmaf(k4.w, value, fmaf(-au4.w, along, w4.w * s[4 * g + 3]));
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) {
+                s[c][4 * g + 0] = fmaf(k4.x, value[c], fmaf(-au4.x, along[c], w4.x * s[c][4 * g + 0]));
+                s[c][4 * g + 1] = fmaf(k4.y, value[c], fmaf(-au4.y, along[c], w4.y * s[c][4 * g + 1]));
+                s[c][4 * g + 2] = fmaf(k4.z, value[c], fmaf(-au4.z, along[c], w4.z * s[c][4 * g + 2]));
+                s[c][4 * g + 3] = fmaf(k4.w, value[c], fmaf(-au4.w, along[c], w4.w * s[c][4 * g + 3]));
+              }
             }
         } else {
 #pragma unroll
-          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
+          for (int g = 0; g < PL / 4; ++g)
             if (4 * g < per_lane) {
               const float4 k4 = *reinterpret_cast<const float4*>(k_lds + 4 * g);
-              s[4 * g + 0] = fmaf(k4.x, value, decay * s[4 * g + 0]);
-              s[4 * g + 1] = fmaf(k4.y, value, decay * s[4 * g + 1]);
-              s[4 * g + 2] = fmaf(k4.z, value, decay * s[4 * g + 2]);
-              s[4 * g + 3] = fmaf(k4.w, value, decay * s[4 * g + 3]);
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) {
+                s[c][4 * g + 0] = fmaf(k4.x, value[c], decay * s[c][4 * g + 0]);
+                s[c][4 * g + 1] = fmaf(k4.y, value[c], decay * s[c][4 * g + 1]);
+                s[c][4 * g + 2] = fmaf(k4.z, value[c], decay * s[c][4 * g + 2]);
+                s[c][4 * g + 3] = fmaf(k4.w, value[c], decay * s[c][4 * g + 3]);
+              }
             }
         }
         if (MODE != LS_LOCAL) {
-          float part[LS_MAX_PER_LANE / 4];
+          float part[CPL][PL / 4];
 #pragma unroll
-          for (int g = 0; g < LS_MAX_PER_LANE / 4; ++g)
-            part[g] = 4 * g < per_lane ? dot4(*reinterpret_cast<const float4*>(q_lds + 4 * g), s + 4 * g) : 0.f;
-          result = column_sum<R_CONST>((part[0] + part[1]) + (part[2] + part[3]), R);
-          if (mine && sub == 0) a.out[(long)(stage_first + tt) * a.out_ld + head * dv + column] = result;
+          for (int g = 0; g < PL / 4; ++g) {
+            const bool live = 4 * g < per_lane;
+            const float4 q4 = live ? *reinterpret_cast<const float4*>(q_lds + 4 * g) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) part[c][g] = dot4(q4, s[c] + 4 * g);
+          }
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) {
+            float sum = part[c][0];
+#pragma unroll
+            for (int g = 1; g < PL / 4; ++g) sum += part[c][g];
+            const float result = column_sum<R_CONST>(sum, R);
+            const int column = column0 + c;
+            if (sub == 0 && column_in_group + c < a.columns && column < dv)
+              a.out[(long)(stage_first + tt) * a.out_ld + head * dv + column] = result;
+          }
         }
       }
     }
   }
-  float* into = state_column;
-  if (MODE == LS_LOCAL) into = a.local + (((long)blockIdx.x * a.H + head) * total_columns + (mine ? column : 0)) * dk;
-  if (mine && (MODE != LS_CHUNK || last_of_lane)) {
 #pragma unroll
-    for (int e = 0; e < LS_MAX_PER_LANE; ++e) {
-      const int channel = channel0 + e;
-      if (e < per_lane && channel < dk) into[channel] = s[e];
+  for (int c = 0; c < CPL; ++c) {
+    const int column = column0 + c;
+    const bool mine = in_group && column_in_group + c < a.columns && column < total_columns;
+    float* into = a.state + (state_head + (mine && column < dv ? column : 0)) * dk;
+    if (MODE == LS_LOCAL) into = a.local + (((long)blockIdx.x * a.H + head) * total_columns + (mine ? column : 0)) * dk;
+    if (mine && (MODE != LS_CHUNK || last_of_lane)) {
+#pragma unroll
+      for (int e = 0; e < PL; ++e) {
+        const int channel = channel0 + e;
+        if (e < per_lane && channel < dk) into[channel] = s[c][e];
+      }
     }
   }
 }
@@ -405,26 +452,38 @@ static int scan_shape(ScanArgs& a, int threads, int total_columns, bool delta, i
   return 0;
 }
 
-#define LS_LAUNCH_R(MODE_, R_, grid_, threads_, lds_)                                                              \
+#define LS_LAUNCH_R(MODE_, R_, PL_, grid_, threads_, lds_)                                                         \
   do {                                                                                                            \
     if (dtype == DT_F32) {                                                                                        \
-      if (delta) linear_state_scan_kernel<float, true, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);          \
-      else linear_state_scan_kernel<float, false, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);               \
+      if (delta) linear_state_scan_kernel<float, true, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);     \
+      else linear_state_scan_kernel<float, false, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);          \
     } else {                                                                                                      \
-      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);         \
-      else linear_state_scan_kernel<bf16_t, false, MODE_, R_><<<grid_, threads_, lds_, stream>>>(a);              \
+      if (delta) linear_state_scan_kernel<bf16_t, true, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);    \
+      else linear_state_scan_kernel<bf16_t, false, MODE_, R_, PL_><<<grid_, threads_, lds_, stream>>>(a);         \
     }                                                                                                             \
   } while (0)
-#define LS_LAUNCH(MODE_, grid_, threads_, lds_)                                                                   \
+// the walk from end to end: one column a lane, up to 16 channels of it
+#define LS_LAUNCH_WHOLE(grid_, threads_, lds_)                                                                    \
   do {                                                                                                            \
     switch (a.R) {                                                                                                \
-      case 1: LS_LAUNCH_R(MODE_, 1, grid_, threads_, lds_); break;                                                \
-      case 2: LS_LAUNCH_R(MODE_, 2, grid_, threads_, lds_); break;                                                \
-      case 4: LS_LAUNCH_R(MODE_, 4, grid_, threads_, lds_); break;                                                \
-      case 8: LS_LAUNCH_R(MODE_, 8, grid_, threads_, lds_); break;                                                \
-      case 16: LS_LAUNCH_R(MODE_, 16, grid_, threads_, lds_); break;                                              \
-      default: LS_LAUNCH_R(MODE_, 0, grid_, threads_, lds_); break;                                               \
+      case 1: LS_LAUNCH_R(LS_WHOLE, 1, 16, grid_, threads_, lds_); break;                                         \
+      case 2: LS_LAUNCH_R(LS_WHOLE, 2, 16, grid_, threads_, lds_); break;                                         \
+      case 4: LS_LAUNCH_R(LS_WHOLE, 4, 16, grid_, threads_, lds_); break;                                         \
+      case 8: LS_LAUNCH_R(LS_WHOLE, 8, 16, grid_, threads_, lds_); break;                                         \
+      default: LS_LAUNCH_R(LS_WHOLE, 0, 16, grid_, threads_, lds_); break;                                        \
     }                                                                                                             \
+  } while (0)
+// the passes over chunks: (lanes a column, channels a lane) as pass_shape chose them
+#define LS_LAUNCH_PASS(MODE_, grid_, threads_, lds_)                                                              \
+  do {                                                                                                            \
+    if (a.per_lane == 4 && a.R == 1) LS_LAUNCH_R(MODE_, 1, 4, grid_, threads_, lds_);                             \
+    else if (a.per_lane == 4 && a.R == 2) LS_LAUNCH_R(MODE_, 2, 4, grid_, threads_, lds_);                        \
+    else if (a.per_lane == 4 && a.R == 4) LS_LAUNCH_R(MODE_, 4, 4, grid_, threads_, lds_);                        \
+    else if (a.per_lane == 4 && a.R == 8) LS_LAUNCH_R(MODE_, 8, 4, grid_, threads_, lds_);                        \
+    else if (a.per_lane == 4 && a.R == 16) LS_LAUNCH_R(MODE_, 16, 4, grid_, threads_, lds_);                      \
+    else if (a.per_lane == 8 && a.R == 16) LS_LAUNCH_R(MODE_, 16, 8, grid_, threads_, lds_);                      \
+    else if (a.R == 16) LS_LAUNCH_R(MODE_, 16, 16, grid_, threads_, lds_);                                        \
+    else LS_LAUNCH_R(MODE_, 0, 16, grid_, threads_, lds_);                                                        \
   } while (0)
 
 extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col, int k_col, int v_col, int removal_col,
@@ -446,7 +505,7 @@ extern "C" int mi_linear_state_scan(const void* u, int dtype, long ld, int q_col
   code = scan_shape(a, threads, dv, delta, max_query_len, &lds, &splits);
   if (code) return code;
   const dim3 grid(lanes, H, splits);
-  LS_LAUNCH(LS_WHOLE, grid, threads, lds);
+  LS_LAUNCH_WHOLE(grid, threads, lds);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -481,19 +540,23 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
   // the passes spread a column over more lanes than the walk from end to end: up to LS_PASS_LANES, four key
   // channels a lane or more, so that a token is a short chain of sums and a workgroup of LS_PASS_THREADS threads
   // still takes 64 columns with one copy of the stage's vectors
+  // and a lane keeps 16 / (channels a lane) neighbouring columns, which share every read of the token's vectors
+  int columns_a_lane = 1;
   {
+    const int channels = dk <= 64 ? 4 : dk <= 128 ? 8 : LS_MAX_PER_LANE;
     int R = 1;
-    while (R * 4 < dk && R < LS_PASS_LANES) R *= 2;
-    while (R * LS_MAX_PER_LANE < dk) R *= 2;
+    while (R * channels < dk) R *= 2;
     a.R = R;
-    a.per_lane = (((dk + R - 1) / R + 3) / 4) * 4;
+    a.per_lane = channels < LS_MAX_PER_LANE ? channels : (((dk + R - 1) / R + 3) / 4) * 4;
+    columns_a_lane = LS_MAX_PER_LANE / channels;
   }
   // local: the chunks' own states (and transitions)
-  code = scan_shape(a, LS_PASS_THREADS, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, delta ? dv + dk : dv, delta, chunk_tokens, &lds, &splits);
   if (code) return code;
-  int threads = ((a.columns * a.R + WAVE - 1) / WAVE) * WAVE;          // no more waves than the columns fill
+  // no more waves than the columns fill
+  int threads = (((a.columns + columns_a_lane - 1) / columns_a_lane * a.R + WAVE - 1) / WAVE) * WAVE;
   if (threads < LS_THREADS) threads = LS_THREADS;
-  LS_LAUNCH(LS_LOCAL, dim3(num_chunks, H, splits), threads, lds);
+  LS_LAUNCH_PASS(LS_LOCAL, dim3(num_chunks, H, splits), threads, lds);
   RETURN_IF_LAUNCH_FAILED();
   // carry: every chunk's starting state
   const int carry_splits = (dv + LS_CARRY_COLUMNS - 1) / LS_CARRY_COLUMNS;
@@ -505,11 +568,11 @@ extern "C" int mi_linear_state_scan_chunked(const void* u, int dtype, long ld, i
   else linear_state_carry_kernel<false><<<dim3(lanes, H, carry_splits), carry_threads, carry_lds, stream>>>(a);
   RETURN_IF_LAUNCH_FAILED();
   // scan: the outputs, and the requests' states behind their last chunks
-  code = scan_shape(a, LS_PASS_THREADS, dv, delta, chunk_tokens, &lds, &splits);
+  code = scan_shape(a, LS_PASS_THREADS * columns_a_lane, dv, delta, chunk_tokens, &lds, &splits);
   if (code) return code;
-  threads = ((a.columns * a.R + WAVE - 1) / WAVE) * WAVE;
+  threads = (((a.columns + columns_a_lane - 1) / columns_a_lane * a.R + WAVE - 1) / WAVE) * WAVE;
   if (threads < LS_THREADS) threads = LS_THREADS;
-  LS_LAUNCH(LS_CHUNK, dim3(num_chunks, H, splits), threads, lds);
+  LS_LAUNCH_PASS(LS_CHUNK, dim3(num_chunks, H, splits), threads, lds);
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -111,7 +111,9 @@ def scan_case(delta, H, dk, dv, lengths, dtype, rotary, seed):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("delta, H, dk, dv, rotary", [
     (False, 3, 16, 16, 16), (False, 2, 24, 40, 12), (False, 1, 64, 128, 0), (False, 2, 40, 8, 40),
-    (True, 2, 16, 16, 0), (True, 3, 24, 24, 0), (True, 1, 64, 64, 0), (True, 2, 72, 72, 0), (True, 1, 130, 130, 0)])
+    (False, 2, 32, 10, 8), (False, 1, 128, 6, 0), (False, 1, 100, 262, 100),
+    (True, 2, 16, 16, 0), (True, 3, 24, 24, 0), (True, 1, 64, 64, 0), (True, 2, 72, 72, 0), (True, 1, 130, 130, 0),
+    (True, 2, 20, 20, 0), (True, 1, 6, 6, 0)])
 def test_scans_walk_lanes_and_chunks_alike(dtype, delta, H, dk, dv, rotary):
     """Lanes of 1, 2, 15, 16, 17 and 70 tokens from states that are not empty, in slots out of order: the walk from
     end to end and the three passes over chunks of 16 tokens against the reference, outputs and states."""
