@@ -382,7 +382,7 @@ extern "C" int mi_add_bias_round(const float* sums, const float* bias, void* out
 //   v = h[r] + scale * delta[r] (the product and the sum in float32);  if no `rows`: h[r] = v;
 //   out[i] = v / sqrt(mean(v^2) + eps) * weight     (out may be null: the add alone).
 // One workgroup a row; a thread keeps its elements of the row in registers (up to SCALED_MAX_ROUNDS * 256 columns)
-// or, for wider rows, in LDS.  The sum of squares is added up in an order that d alone fixes.
+// or, for wider rows, in LDS.  The sum of squares is added up in an order that d and the workgroup's size fix.
 #define SCALED_MAX_ROUNDS 8
 template <typename TD, typename TO, bool IN_LDS>
 __global__ void __launch_bounds__(1024)
@@ -436,8 +436,9 @@ extern "C" int mi_add_scaled_rmsnorm(float* h, const void* delta, int delta_dtyp
                                      const float* weight, float eps, void* out, int out_dtype, const int* rows,
                                      int n_rows, int d, hipStream_t stream) {
   if (!h || !delta || !scale || !weight || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
-  // a narrow row takes 256 threads; a wide one 1,024, so that a step of few rows still has waves to hide its waits
-  const int threads = d > 2048 ? 1024 : 256;
+  // 256 threads a row; a wide row of a step of few rows 1,024, so that the step still has waves to hide its waits
+  // (a prompt's thousands of rows fill the GPU as they are: 26 us against 19 for 2,048 rows of 3,072 with the wide ones)
+  const int threads = (d > 2048 && n_rows <= 512) ? 1024 : 256;
   const bool in_lds = d > threads * SCALED_MAX_ROUNDS;
   if (in_lds && (size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
   const size_t lds = in_lds ? (size_t)d * sizeof(float) : 0;
@@ -495,7 +496,7 @@ polynorm_kernel(const T* __restrict__ z, long ld, const float* __restrict__ coef
 extern "C" int mi_polynorm(const void* z, int dtype, long ld, const float* coefficients, float eps, void* out,
                            long out_ld, int T, int I, hipStream_t stream) {
   if (!z || !coefficients || !out || T <= 0 || I <= 0 || ld < I || out_ld < I) return ERR_BAD_ARGUMENT;
-  const int threads = I > 2048 ? 1024 : 256;
+  const int threads = (I > 2048 && T <= 512) ? 1024 : 256;          // as add_scaled_rmsnorm: wide rows of few-row steps
   if (dtype == DT_F32)
     polynorm_kernel<float><<<T, threads, 0, stream>>>((const float*)z, ld, coefficients, eps, (float*)out, out_ld, I);
   else if (dtype == DT_BF16)
