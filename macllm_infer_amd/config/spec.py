@@ -62,6 +62,32 @@ class RmsNormSpec:
 
 
 @dataclass(frozen=True)
+class InterleavedRopeSpec:
+    """Rotary position encoding whose pairs are neighbours: dimension 2i turns with dimension 2i + 1, i below
+    ``rotary_dim`` / 2, by the angle position * theta^(-2i / rotary_dim); dimensions from ``rotary_dim`` on pass
+    unchanged."""
+    theta: float
+    rotary_dim: int
+    kind: str = "rope_interleaved"
+
+    def validate(self, head_dim: int) -> None:
+        _require(self.theta > 0 and self.theta == self.theta and self.theta != float("inf"),
+                 f"rope theta must be finite and positive, got {self.theta}")
+        _require(0 < self.rotary_dim <= head_dim and self.rotary_dim % 2 == 0,
+                 f"rotary_dim {self.rotary_dim} must be even and in 2..={head_dim}")
+
+
+@dataclass(frozen=True)
+class LayerNormSpec:
+    """y = (x - mean) / sqrt(variance + eps) * weight + bias, the variance the mean of the squared deviations."""
+    eps: float
+    kind: str = "layernorm"
+
+    def validate(self) -> None:
+        _require(self.eps > 0, f"norm eps must be positive, got {self.eps}")
+
+
+@dataclass(frozen=True)
 class LogDistanceBiasSpec:
     """No rotation; the score of a key at distance n behind the query loses r1 * ln(1 + r2 * n), with r1 and
     r2 learned numbers of each query head (tensors ``r1`` and ``r2`` of the mixer)."""
@@ -114,6 +140,106 @@ class AttentionSpec:
         _require(self.scale > 0, "attention scale must be positive")
         _require(self.window is None or self.window > 0, "attention window must be positive")
         self.position.validate(self.head_dim)
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal softmax attention whose queries, keys and values come through low-rank latents.
+
+    Queries: c_q = RMSNorm(W_dq h) [``q_rank``], q = W_uq c_q, per head ``head_dim`` plain dimensions followed by
+    ``rope_dim`` turned ones.  Keys and values: W_dkv h gives ``kv_rank`` + ``rope_dim`` numbers; the first
+    ``kv_rank``, RMS-normed, are the latent c, the rest is one turned key part shared by all heads.  A head's plain
+    key is W_uk c, its value W_uv c (``value_dim`` wide); score = (q_plain . k_plain + q_turned . k_turned) *
+    ``scale``.  The cache holds c and the turned key part of a token, nothing per head.  ``position`` turns the
+    ``rope_dim`` part of q and k."""
+    num_heads: int
+    head_dim: int
+    rope_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    position: object = field(default_factory=NoPositionSpec)
+    window: Optional[int] = None
+    kind: str = "latent_attention"
+
+    @property
+    def cached_key_dim(self) -> int:
+        """What a token's key is in the cache: its latent and the turned part."""
+        return self.kv_rank + self.rope_dim
+
+    def validate(self) -> None:
+        for name in ("num_heads", "head_dim", "value_dim", "q_rank", "kv_rank"):
+            _require(getattr(self, name) > 0, f"latent attention {name} must be positive")
+        _require(self.rope_dim >= 0, "latent attention rope_dim cannot be negative")
+        _require(self.scale > 0, "attention scale must be positive")
+        _require(self.norm_eps > 0, "latent attention norm eps must be positive")
+        _require(self.window is None or self.window > 0, "attention window must be positive")
+        if self.rope_dim:
+            self.position.validate(self.rope_dim)
+
+
+@dataclass(frozen=True)
+class ClampedGLUSpec:
+    """The activation of a gated feed-forward with clamped branches: g = min(gate, limit),
+    u = clamp(up, -limit, limit), y = g * sigmoid(alpha g) * (u + up_offset)."""
+    limit: float
+    alpha: float = 1.702
+    up_offset: float = 1.0
+
+    def validate(self) -> None:
+        _require(self.limit > 0 and self.limit == self.limit, "the activation's limit must be positive")
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A mixture of ``num_experts`` small gated feed-forwards (``expert_size`` wide, no biases) of which a token
+    uses ``top_k``, and optionally a shared one (``shared_size`` wide) that every token uses, times
+    sigmoid(w_sg . x).  Router: s = softmax(W_router x) over all experts in float32; the ``top_k`` largest of
+    s + correction are chosen; their weights are their s divided by the sum of the chosen s (+ ``weight_eps``),
+    times ``route_scale``."""
+    num_experts: int
+    top_k: int
+    expert_size: int
+    activation: ClampedGLUSpec
+    route_scale: float = 1.0
+    weight_eps: float = 1e-20
+    shared_size: Optional[int] = None
+    shared_activation: Optional[ClampedGLUSpec] = None
+    kind: str = "routed_experts"
+
+    def validate(self) -> None:
+        _require(self.num_experts > 0 and self.expert_size > 0, "the experts' number and width must be positive")
+        _require(0 < self.top_k <= self.num_experts,
+                 f"a token uses {self.top_k} experts of {self.num_experts}")
+        self.activation.validate()
+        if self.shared_size is not None:
+            _require(self.shared_size > 0 and self.shared_activation is not None,
+                     "a shared expert needs a positive width and an activation")
+            self.shared_activation.validate()
+
+
+@dataclass(frozen=True)
+class HashedBigramSpec:
+    """A second embedding row for every token, picked by a hash of the token and the one before it: row
+    (previous * mul_prev + token * mul_cur) mod ``buckets`` of a table of ``buckets`` + 1 rows; a sequence's
+    first token takes the last row.  The previous token is part of a request's state."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+    def validate(self) -> None:
+        _require(self.buckets > 0, "the bigram table needs at least one bucket")
+
+
+@dataclass(frozen=True)
+class StreamInjection:
+    """What is added to the residual stream right before a schedule entry runs: the embedding output once more
+    (``embedding``), and row ``row`` of the tensor ``vector_name`` [rows, hidden] (None: no vector)."""
+    embedding: bool = False
+    vector_name: Optional[str] = None
+    row: int = 0
 
 
 @dataclass(frozen=True)
@@ -260,6 +386,8 @@ class LayerSpec:
     # before it is added to the residual stream (None: no such scale)
     mixer_scale_name: Optional[str] = None
     ffn_scale_name: Optional[str] = None
+    # one number that multiplies every branch where it joins the stream (x <- x + m * branch), applied in float32
+    branch_multiplier: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -270,6 +398,7 @@ class ScheduleEntry:
     of its own (only mixers whose cache is token-proportional can do that)."""
     layer: int
     kv_from: Optional[int] = None
+    before: Optional[StreamInjection] = None      # added to the stream right before this run
 
 
 @dataclass(frozen=True)
@@ -286,6 +415,10 @@ class ModelSpec:
     logit_multiplier: float = 1.0
     # logits <- cap * tanh(logits / cap) after their scaling (src/decoder.rs:3349-3355, 4791-4796); None: no cap
     logit_softcap: Optional[float] = None
+    bigram: Optional[HashedBigramSpec] = None      # a hashed bigram row added to every token's embedding
+    bigram_name: str = "bigram"
+    # tensors [rows, hidden] that schedule entries name (``StreamInjection.vector_name``): (name, rows)
+    injected_vectors: Tuple[Tuple[str, int], ...] = ()
     embedding_name: str = "model.embed_tokens"
     final_norm_name: str = "model.norm"
     lm_head_name: str = "lm_head"
@@ -318,6 +451,14 @@ class ModelSpec:
         _require(self.logit_softcap is None or (0 < self.logit_softcap < float("inf")),
                  f"the cap on the logits must be finite and positive, got {self.logit_softcap}")
         self.final_norm.validate()
+        if self.bigram is not None:
+            self.bigram.validate()
+        vectors = dict(self.injected_vectors)
+        for index, entry in enumerate(self.schedule):
+            if entry.before is not None and entry.before.vector_name is not None:
+                _require(entry.before.vector_name in vectors
+                         and 0 <= entry.before.row < vectors[entry.before.vector_name],
+                         f"schedule entry {index} adds a row of a vector table that the model does not have")
         for layer in self.layers:
             _require(len(layer.mixers) > 0, f"layer {layer.prefix} has no mixer")
             names = [slot.name for slot in layer.mixers]

@@ -10,7 +10,8 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..kernels import ops
-from ..parts.base import BuildContext, Residual, part_class
+from ..cache.manager import StateNeed
+from ..parts.base import BuildContext, Residual, RowVector, WeightedBranch, part_class
 from ..parts.block import arrangement_class
 from ..weights.loader import Expect
 
@@ -22,6 +23,9 @@ from ..weights.loader import Expect
 # second, and 1,333 on a 261,120 x 5,120 head that streams in 450.)
 HEAD_SKINNY_ROWS = 8
 
+# the cache key of what the model itself keeps for a request, beside its mixers' (entry, mixer name) keys
+MODEL_STATE = ("model", "embedding")
+
 
 class DecoderModel:
     @staticmethod
@@ -29,6 +33,10 @@ class DecoderModel:
         """Every tensor the model binds, by exact name with its shape
         (name tables: src/architecture.rs:1595-1647)."""
         out = [Expect(f"{spec.embedding_name}.weight", ((spec.vocab_size, spec.hidden_size),), init="embedding")]
+        if spec.bigram is not None:
+            out.append(Expect(f"{spec.bigram_name}.weight", ((spec.bigram.buckets + 1, spec.hidden_size),), init="embedding"))
+        for name, rows in spec.injected_vectors:
+            out.append(Expect(name, ((rows, spec.hidden_size),), init="bias"))
         for layer in spec.layers:
             out += arrangement_class(layer.arrangement).expected_tensors(layer, spec.hidden_size)
         out += part_class(spec.final_norm).expected_tensors(spec.final_norm, spec.final_norm_name, spec.hidden_size)
@@ -74,6 +82,8 @@ class DecoderModel:
                 needs[key] = list(part_class(slot.spec).cache_needs(slot.spec))
                 if entry.kv_from is not None and any(getattr(need, "token_proportional", False) for need in needs[key]):
                     shared[key] = (entry.kv_from, slot.name)
+        if spec.bigram is not None:                       # the token before a step's first one
+            needs[MODEL_STATE] = [StateNeed("previous_token", (1,), torch.int32)]
         return needs, shared
 
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], build: BuildContext):
@@ -84,6 +94,14 @@ class DecoderModel:
         if build.dtype == torch.float32:
             table = table.to(torch.float32)
         self.embedding = table.contiguous().to(build.device)
+        self.bigram = None
+        if spec.bigram is not None:
+            table = tensors[f"{spec.bigram_name}.weight"]
+            self.bigram = (table.to(torch.float32) if build.dtype == torch.float32 else table).contiguous().to(build.device)
+        # the vectors that schedule entries add to the stream, float32 on the device
+        self.injected = {name: tensors[name].to(torch.float32).contiguous().to(build.device)
+                         for name, _ in spec.injected_vectors}
+        self._keeps_embedding = any(entry.before is not None and entry.before.embedding for entry in spec.schedule)
         self.blocks = [arrangement_class(layer.arrangement)(layer, tensors, build) for layer in spec.layers]
         for block in self.blocks:                    # what a layer decides by timing itself among the others
             tune = getattr(block, "tune", None)
@@ -139,10 +157,25 @@ class DecoderModel:
         [wanted, vocab] at ``step.want_rows`` (empty tensor when nothing is wanted)."""
         spec = self.spec
         h = torch.empty((step.num_tokens, spec.hidden_size), dtype=torch.float32, device=self.build.device)
-        ops.embed(step.token_ids, self.embedding, spec.embedding_multiplier, h)
+        if self.bigram is None:
+            ops.embed(step.token_ids, self.embedding, spec.embedding_multiplier, h)
+        else:
+            ops.embed_bigram(step.token_ids, self.embedding, spec.embedding_multiplier, self.bigram, spec.bigram.buckets,
+                             spec.bigram.mul_prev, spec.bigram.mul_cur, step.positions, step.lane_of_token,
+                             step.cu_seqlens, step.slot_ids, cache.entry(MODEL_STATE).states["previous_token"], h)
+        embedded = h.clone() if self._keeps_embedding else None
         residual = Residual(h)
         for index, entry in enumerate(spec.schedule):
             block = self.blocks[entry.layer]
+            if entry.before is not None:
+                # what joins the stream before this run waits with the branches of the run before it: the run's
+                # first norm adds them all in its own launch
+                added = list(residual.pending)
+                if entry.before.embedding:
+                    added.append(WeightedBranch(embedded, 1.0))
+                if entry.before.vector_name is not None:
+                    added.append(RowVector(self.injected[entry.before.vector_name][entry.before.row]))
+                residual.pending = added
             caches = {name: cache.entry((index, name)) for name, _ in block.mixers}
             residual.next_norm = self._next_norms[index]
             block.forward(residual, step, caches)

@@ -14,6 +14,7 @@ CONV_MAX_TAPS = 16                # CONV_MAX_K in mamba2.hip: the taps of a chan
 SCAN_MAX_STATE = 512              # WAVE * SCAN_MAX_PER_THREAD in mamba2.hip: a state row over one wave
 LINEAR_STATE_MAX_KEY_DIM = 1024   # LS_MAX_PER_LANE * WAVE in linear_state.hip: a state column over one wave
 NORM_MAX_WIDTH = 16384            # 64 KiB of LDS hold a float32 row in common.hip's norm
+MOE_MAX_EXPERTS = 1024            # MOE_MAX_EXPERTS in moe.hip: the experts' counts in LDS, 16 scores a lane
 GRID_MOST = 65535                 # heads, groups or lanes that index a launch's y or z dimension
 
 

@@ -43,6 +43,31 @@ _SIGNATURES = {
         "mi_add_scaled_rmsnorm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
                                   _c_ptr],
         "mi_polynorm": [_c_ptr, _c_int, _c_long, _c_ptr, _c_float, _c_ptr, _c_long, _c_int, _c_int, _c_ptr],
+        "mi_embed_bigram": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_long, _c_long, _c_ptr, _c_ptr, _c_ptr,
+                            _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+        "mi_stream_add": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_add_layernorm": [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_float, _c_ptr,
+                             _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+        "mi_clamped_glu": [_c_ptr, _c_int, _c_long, _c_ptr, _c_long, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr],
+    },
+    "latent": {
+        "mi_latent_prepare": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr,
+                              _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_long, _c_ptr],
+        "mi_rotate_heads": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
+                            _c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr],
+        "mi_head_gemm": [_c_ptr, _c_int, _c_long, _c_long, _c_ptr, _c_long, _c_long, _c_ptr, _c_long, _c_long, _c_int,
+                         _c_int, _c_int, _c_int, _c_ptr],
+        "mi_latent_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int,
+                                _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+    },
+    "moe": {
+        "mi_moe_route": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_moe_plan": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_moe_expert_gemm": [_c_ptr, _c_int, _c_long, _c_int, _c_ptr, _c_long, _c_long, _c_int, _c_int, _c_ptr, _c_ptr,
+                               _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr, _c_int, _c_long,
+                               _c_ptr],
+        "mi_moe_combine": [_c_ptr, _c_long, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_long, _c_ptr, _c_ptr, _c_int, _c_int,
+                           _c_ptr],
     },
     "linear_state": {
         "mi_linear_state_scan": [_c_ptr, _c_int, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
@@ -335,6 +360,271 @@ def polynorm(z: torch.Tensor, coefficients: torch.Tensor, eps: float, out: torch
           and coefficients.is_contiguous(), "polynorm: coefficients must be float32 [4] on the GPU")
     _check(_fn("common", "mi_polynorm")(_p(z), _dt(z), ld, _p(coefficients), float(eps), _p(out), out_ld, z.shape[0],
                                         z.shape[1], _stream()), "polynorm")
+
+
+# --------------------------------------------------------------------------- bigram embedding, layer norm, clamped GLU
+def embed_bigram(token_ids: torch.Tensor, table: torch.Tensor, multiplier: float, bigram: torch.Tensor, buckets: int,
+                 mul_prev: int, mul_cur: int, positions: torch.Tensor, lane_of_token: torch.Tensor,
+                 cu_seqlens: torch.Tensor, slot_ids: torch.Tensor, previous: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t] = table[token] * multiplier + bigram[row]: row = (token before * mul_prev + token * mul_cur) mod
+    ``buckets``, or ``buckets`` (the table's last row) at position 0.  The token before a lane's first one is
+    ``previous[slot of the lane]`` (int32 [slots, 1]); a second launch then leaves the lane's last token there."""
+    T, d = out.shape
+    for name, tensor in (("token_ids", token_ids), ("positions", positions), ("lane_of_token", lane_of_token),
+                         ("cu_seqlens", cu_seqlens), ("slot_ids", slot_ids), ("previous", previous)):
+        _i32(tensor, name)
+    lanes = slot_ids.numel()
+    _need(token_ids.numel() == T and positions.numel() == T and lane_of_token.numel() == T
+          and cu_seqlens.numel() == lanes + 1, "embed_bigram: the step's arrays do not fit its tokens and lanes")
+    _need(table.dim() == 2 and table.shape[1] == d and table.is_contiguous() and bigram.shape == (buckets + 1, d)
+          and bigram.is_contiguous() and bigram.dtype == table.dtype, "embed_bigram: tables do not fit")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed_bigram: out must be contiguous float32")
+    _check(_fn("common", "mi_embed_bigram")(
+        _p(token_ids), _p(table), _dt(table), float(multiplier), _p(bigram), int(buckets), int(mul_prev), int(mul_cur),
+        _p(positions), _p(lane_of_token), _p(cu_seqlens), _p(slot_ids), _p(previous), _p(out), T, d, lanes, _stream()),
+        "embed_bigram")
+
+
+def stream_add(h: torch.Tensor, rows: Optional[torch.Tensor], factor: float, vector: Optional[torch.Tensor]) -> None:
+    """h += factor * rows (+ vector on every row), in float32, in place."""
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and h.is_cuda,
+          "stream_add: h must be contiguous float32 [T, d]")
+    T, d = h.shape
+    _need(rows is None or (rows.shape == h.shape and rows.is_contiguous()), "stream_add: rows must be contiguous [T, d]")
+    _need(vector is None or (vector.dtype == torch.float32 and vector.numel() == d and vector.is_contiguous()),
+          "stream_add: the vector must be float32 [d]")
+    if rows is None and vector is None:
+        return
+    _check(_fn("common", "mi_stream_add")(_p(h), _p(rows), _dt(rows) if rows is not None else DT_F32, float(factor),
+                                          _p(vector), T, d, _stream()), "stream_add")
+
+
+def add_layernorm(h: torch.Tensor, branches: Sequence[tuple], vector: Optional[torch.Tensor], weight: torch.Tensor,
+                  bias: torch.Tensor, eps: float, out: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+    """h += sum of factor * branch over ``branches`` [(tensor [T, d], factor)] (at most three) + ``vector`` [d]
+    (float32, in place); out = (h - mean) / sqrt(variance + eps) * weight + bias, statistics in float32, the
+    variance from the deviations.  With ``rows`` only those rows are read, ``out[i]`` gets row ``rows[i]`` and
+    ``h`` is left as it is."""
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous() and h.is_cuda,
+          "add_layernorm: h must be contiguous float32 [T, d]")
+    T, d = h.shape
+    _need(len(branches) <= 3, "add_layernorm: at most three branches")
+    for tensor, _ in branches:
+        _need(tensor.shape == h.shape and tensor.is_contiguous(), "add_layernorm: branches must be contiguous [T, d]")
+    for name, one in (("weight", weight), ("bias", bias)):
+        _need(one.dtype == torch.float32 and one.numel() == d and one.is_contiguous(), f"add_layernorm: {name} must be float32 [d]")
+    _need(vector is None or (vector.dtype == torch.float32 and vector.numel() == d and vector.is_contiguous()),
+          "add_layernorm: the vector must be float32 [d]")
+    n_rows = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n_rows = rows.numel()
+        _need(out is not None, "add_layernorm: a gather needs somewhere to put its rows")
+    if out is not None:
+        _need(out.shape == (n_rows, d) and out.is_contiguous(), "add_layernorm: out must be contiguous [rows, d]")
+    if n_rows == 0:
+        return
+    flat = []
+    for index in range(3):
+        if index < len(branches):
+            tensor, factor = branches[index]
+            flat += [_p(tensor), _dt(tensor), float(factor)]
+        else:
+            flat += [None, DT_F32, 0.0]
+    _check(_fn("common", "mi_add_layernorm")(
+        _p(h), *flat, _p(vector), _p(weight), _p(bias), float(eps), _p(out), _dt(out) if out is not None else DT_F32,
+        _p(rows), n_rows, d, _stream()), "add_layernorm", f"(d={d})")
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, up_offset: float, out: torch.Tensor) -> None:
+    """out = g * sigmoid(alpha g) * (u + up_offset) with g = min(gate, limit), u = clamp(up, -limit, limit); a row of
+    ``gate_up`` holds [gate | up]."""
+    ld = _row_major(gate_up, "gate_up")
+    out_ld = _row_major(out, "out")
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and out.shape == (T, two_i // 2) and out.dtype == gate_up.dtype,
+          "clamped_glu: out must be [T, I] of the input's dtype")
+    _check(_fn("common", "mi_clamped_glu")(_p(gate_up), _dt(gate_up), ld, _p(out), out_ld, T, two_i // 2, float(limit),
+                                           float(alpha), float(up_offset), _stream()), "clamped_glu")
+
+
+# --------------------------------------------------------------------------- latent attention
+def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rope_dim: int, q_norm: torch.Tensor,
+                   kv_norm: torch.Tensor, eps: float, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                   rotary_dim: int, interleaved: bool, slot_mapping: Optional[torch.Tensor],
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], query_latent: torch.Tensor) -> None:
+    """From a token's down-projected row [query latent | key/value latent | key part to turn]: the query latent's
+    RMS norm (times ``q_norm``) into ``query_latent``; the key/value latent's RMS norm (times ``kv_norm``) and the
+    key part, its first ``rotary_dim`` dimensions turned by the token's position, into the token's cache cell: K
+    pages [pages, 1, page_size, kv_rank + rope_dim] get [latent | turned part], V pages [pages, 1, kv_rank,
+    page_size] the latent.  Norms, angles and the turn are float32.  Without ``slot_mapping`` nothing is stored."""
+    ld = _row_major(down, "down")
+    T = down.shape[0]
+    _need(down.shape[1] >= q_rank + kv_rank + rope_dim, "latent_prepare: the projected rows are too narrow")
+    _i32(positions, "positions")
+    _need(positions.numel() == T, "latent_prepare: one position per token")
+    for name, vector, size in (("q_norm", q_norm, q_rank), ("kv_norm", kv_norm, kv_rank)):
+        _need(vector.dtype == torch.float32 and vector.numel() == size and vector.is_contiguous() and vector.is_cuda,
+              f"latent_prepare: {name} must be float32 [{size}] on the GPU")
+    turned = int(rotary_dim) if inv_freq is not None else 0
+    _need(turned % 2 == 0 and turned <= rope_dim, "latent_prepare: the turned dimensions are pairs within the key part")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == turned // 2 and inv_freq.is_cuda,
+              "latent_prepare: inv_freq must be float32 [rotary_dim / 2]")
+    q_ld = _row_major(query_latent, "query_latent")
+    _need(query_latent.shape == (T, q_rank) and query_latent.dtype == down.dtype, "latent_prepare: query_latent must be [T, q_rank]")
+    page_stride, page_size = 0, 0
+    if slot_mapping is not None:
+        _i32(slot_mapping, "slot_mapping")
+        _need(slot_mapping.numel() == T, "latent_prepare: one cache cell per token")
+        page_stride, page_size = _cache_view(k_cache, v_cache, 1, kv_rank + rope_dim, down.dtype, kv_rank)
+    _check(_fn("latent", "mi_latent_prepare")(
+        _p(down), _dt(down), ld, T, q_rank, kv_rank, rope_dim, _p(q_norm), _p(kv_norm), float(eps), _p(positions),
+        _p(inv_freq), turned, 1 if interleaved else 0, _p(slot_mapping),
+        _p(k_cache) if slot_mapping is not None else None, _p(v_cache) if slot_mapping is not None else None,
+        page_stride, page_size, _p(query_latent), q_ld, _stream()), "latent_prepare")
+
+
+def rotate_heads(x: torch.Tensor, col: int, head_stride: int, num_heads: int, width: int, positions: torch.Tensor,
+                 inv_freq: Optional[torch.Tensor], rotary_dim: int, interleaved: bool, out: torch.Tensor, out_col: int,
+                 out_head_stride: int) -> None:
+    """out[t, out_col + h * out_head_stride + j] = the turned x[t, col + h * head_stride + j], j below ``width``: the
+    first ``rotary_dim`` of the ``width`` dimensions turned in pairs by the token's position, the rest copied."""
+    ld = _row_major(x, "x")
+    out_ld = _row_major(out, "out")
+    T = x.shape[0]
+    _i32(positions, "positions")
+    turned = int(rotary_dim) if inv_freq is not None else 0
+    _need(out.shape[0] == T and positions.numel() == T and out.dtype == x.dtype and turned % 2 == 0 and turned <= width
+          and col + (num_heads - 1) * head_stride + width <= x.shape[1]
+          and out_col + (num_heads - 1) * out_head_stride + width <= out.shape[1], "rotate_heads: shapes do not fit")
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == turned // 2 and inv_freq.is_cuda,
+              "rotate_heads: inv_freq must be float32 [rotary_dim / 2]")
+    _check(_fn("latent", "mi_rotate_heads")(
+        _p(x), _dt(x), ld, int(col), int(head_stride), num_heads, width, _p(positions), _p(inv_freq), turned,
+        1 if interleaved else 0, _p(out), out_ld, int(out_col), int(out_head_stride), T, _stream()), "rotate_heads")
+
+
+def head_linear(x: torch.Tensor, x_col: int, x_head_stride: int, weight: torch.Tensor, out: torch.Tensor, out_col: int,
+                out_head_stride: int) -> None:
+    """One product per head: out[:, out_col + h * out_head_stride : + N] = x[:, x_col + h * x_head_stride : + K] .
+    weight[h]^T, ``weight`` [heads, N, K], float32 sums on the matrix cores (float32 operands: true 32-bit)."""
+    ldx = _row_major(x, "x")
+    ldo = _row_major(out, "out")
+    _need(weight.dim() == 3 and weight.is_contiguous() and weight.is_cuda, "head_linear: weight must be contiguous [heads, N, K]")
+    heads, N, K = weight.shape
+    T = x.shape[0]
+    _need(out.shape[0] == T and x_col + (heads - 1) * x_head_stride + K <= x.shape[1]
+          and out_col + (heads - 1) * out_head_stride + N <= out.shape[1], "head_linear: shapes do not fit")
+    rows = x if x.dtype == weight.dtype else x.to(weight.dtype)
+    target = out if out.dtype == weight.dtype else torch.empty(out.shape, dtype=weight.dtype, device=out.device)
+    if rows is not x:
+        ldx = _row_major(rows, "x")
+    if target is not out:
+        ldo = _row_major(target, "out")
+    _check(_fn("latent", "mi_head_gemm")(
+        _p(rows), _dt(rows), ldx, int(x_col), _p(weight), int(x_head_stride), int(out_head_stride), _p(target), ldo,
+        int(out_col), T, N, K, heads, _stream()), "head_linear", f"(N={N}, K={K})")
+    if target is not out:
+        width = (heads - 1) * out_head_stride + N
+        out[:, out_col:out_col + width] = target[:, out_col:out_col + width].to(out.dtype)
+
+
+def latent_attention_supported(dtype, num_heads: int, kv_rank: int, rope_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core kernel for prompt portions of latent attention covers this geometry."""
+    return False
+
+
+# --------------------------------------------------------------------------- routed experts
+MOE_TILE_ROWS = 16
+
+
+def moe_route(logits: torch.Tensor, num_experts: int, top_k: int, correction: torch.Tensor, scale: float, eps: float,
+              shared_gate: bool):
+    """From float32 router logits [T, >= num_experts (+ 1)]: s = softmax over the experts; the ``top_k`` largest of
+    s + correction (ties to the lower number) are the token's experts (int32 [T, top_k]), their weights (float32
+    [T, top_k]) s / (sum of the chosen s + eps) * scale; with ``shared_gate`` also sigmoid of column
+    ``num_experts`` (float32 [T]), else None."""
+    ld = _row_major(logits, "logits")
+    T = logits.shape[0]
+    _need(logits.dtype == torch.float32 and logits.shape[1] >= num_experts + (1 if shared_gate else 0),
+          "moe_route: float32 logits of every expert")
+    _need(correction.dtype == torch.float32 and correction.numel() == num_experts and correction.is_cuda,
+          "moe_route: the correction must be float32 [experts] on the GPU")
+    _need(0 < top_k <= num_experts, "moe_route: a token uses at least one and at most all experts")
+    chosen = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top_k), dtype=torch.float32, device=logits.device)
+    gate = torch.empty((T,), dtype=torch.float32, device=logits.device) if shared_gate else None
+    _check(_fn("moe", "mi_moe_route")(_p(logits), ld, T, num_experts, top_k, _p(correction), float(scale), float(eps),
+                                      _p(chosen), _p(weights), _p(gate), _stream()), "moe_route", f"(experts={num_experts})")
+    return chosen, weights, gate
+
+
+class MoePlan:
+    """The rows of a step grouped by expert, on the device: ``source`` int32 [capacity] = the token whose row
+    stands at a place (-1: padding), ``place`` int32 [T * top_k] = where a token's choice stands, ``tile_expert``
+    int32 [capacity / pad] = the expert of every tile of ``pad`` places (-1: an unused tile).  Every expert's rows
+    start a tile; ``capacity`` depends on the number of tokens alone."""
+
+    def __init__(self, chosen: torch.Tensor, num_experts: int, pad: int = MOE_TILE_ROWS):
+        _i32(chosen, "chosen")
+        tokens, top_k = chosen.shape
+        self.pad, self.tokens, self.top_k = pad, tokens, top_k
+        self.capacity = -(-(tokens * top_k + num_experts * (pad - 1)) // pad) * pad
+        device = chosen.device
+        self.source = torch.empty((self.capacity,), dtype=torch.int32, device=device)
+        self.place = torch.empty((tokens * top_k,), dtype=torch.int32, device=device)
+        self.tile_expert = torch.empty((self.capacity // pad,), dtype=torch.int32, device=device)
+        ranks = torch.empty((tokens * top_k,), dtype=torch.int32, device=device)
+        _check(_fn("moe", "mi_moe_plan")(_p(chosen), tokens * top_k, top_k, num_experts, pad, self.capacity,
+                                         _p(self.source), _p(self.place), _p(self.tile_expert), _p(ranks), _stream()),
+               "moe_plan", f"(experts={num_experts})")
+
+
+def moe_plan(chosen: torch.Tensor, num_experts: int) -> MoePlan:
+    return MoePlan(chosen, num_experts)
+
+
+def moe_expert_gemm(x: torch.Tensor, plan: MoePlan, weight: torch.Tensor, out: torch.Tensor, gather: bool, glu) -> None:
+    """The grouped product of a plan's rows with their experts' matrices ``weight`` [experts, N, K]: the row at a
+    place is ``x[source[place]]`` (``gather``) or ``x[place]``; out[place] = weight[expert] . row, or with ``glu``
+    (limit, alpha, up_offset; N = 2 I, gate rows then up rows) the clamped gated activation of the two halves,
+    [capacity, I].  Float32 sums on the matrix cores; float32 operands give a true 32-bit product."""
+    ldx = _row_major(x, "x")
+    ldo = _row_major(out, "out")
+    _need(weight.dim() == 3 and weight.is_contiguous() and weight.is_cuda and x.dtype == weight.dtype,
+          "moe_expert_gemm: weight must be contiguous [experts, N, K] of the rows' dtype")
+    experts, N, K = weight.shape
+    width = N // 2 if glu is not None else N
+    _need(x.shape[1] == K and out.shape == (plan.capacity, width) and (gather or x.shape[0] == plan.capacity)
+          and (not gather or x.shape[0] == plan.tokens), "moe_expert_gemm: shapes do not fit the plan")
+    _check(_fn("moe", "mi_moe_expert_gemm")(
+        _p(x), _dt(x), ldx, x.shape[0], _p(weight), N * K, K, N, K, _p(plan.source), _p(plan.tile_expert),
+        plan.tile_expert.numel(), plan.pad, 1 if gather else 0, 1 if glu is not None else 0,
+        float(glu.limit) if glu is not None else 0.0, float(glu.alpha) if glu is not None else 0.0,
+        float(glu.up_offset) if glu is not None else 0.0, _p(out), _dt(out), ldo, _stream()),
+        "moe_expert_gemm", f"(N={N}, K={K})")
+
+
+def moe_combine(down: torch.Tensor, plan: MoePlan, weights: torch.Tensor, shared_rows: Optional[torch.Tensor],
+                shared_gate: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """out[t] = sum over the token's choices k, in their order, of weights[t, k] * down[place[t, k]]
+    (+ shared_gate[t] * shared_rows[t]), float32."""
+    T, d = out.shape
+    ld = _row_major(down, "down")
+    _need(down.dtype == torch.float32 and out.dtype == torch.float32 and out.is_contiguous() and down.shape[1] == d
+          and weights.dtype == torch.float32 and weights.shape == (T, plan.top_k) and weights.is_contiguous()
+          and T == plan.tokens, "moe_combine: shapes do not fit the plan")
+    shared_ld = 0
+    if shared_rows is not None:
+        shared_ld = _row_major(shared_rows, "shared_rows")
+        _need(shared_rows.shape == (T, d) and shared_gate is not None and shared_gate.dtype == torch.float32
+              and shared_gate.numel() == T, "moe_combine: the shared rows and their gate do not fit")
+    _check(_fn("moe", "mi_moe_combine")(
+        _p(down), ld, _p(plan.place), _p(weights), plan.top_k, _p(shared_rows),
+        _dt(shared_rows) if shared_rows is not None else DT_F32, shared_ld, _p(shared_gate), _p(out), T, d, _stream()),
+        "moe_combine")
 
 
 # --------------------------------------------------------------------------- mixers with a matrix-valued state

@@ -1,11 +1,13 @@
 from .base import BuildContext, FeedForward, Mixer, Part, Residual, part_class, register_part
 from .block import ParallelPreNormBlock, arrangement_class, register_arrangement, register_fusion
 from .linear import Linear
-from .norm import RmsNorm
-from .position import LogDistanceBias, NoPosition, PositionEncoding, Rope
+from .norm import LayerNorm, RmsNorm
+from .position import InterleavedRope, LogDistanceBias, NoPosition, PositionEncoding, Rope
 from .attention import Attention
+from .latent_attention import LatentAttention
 from .mamba2 import Mamba2
 from .ffn import PolyNormFFN, SwiGLU
+from .moe import RoutedExperts
 from .linear_state import GeneralDelta, Retention
 from . import fused          # registers the fast paths of the layer arrangements
 from .fused import FastPathDeclined

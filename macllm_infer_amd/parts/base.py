@@ -80,9 +80,23 @@ class ScaledBranch:
     scale: torch.Tensor
 
 
+@dataclass
+class WeightedBranch:
+    """A branch output [T, d] (float32 or the activation dtype) that is multiplied by one number, ``factor``, in
+    float32 where it is added to the residual stream."""
+    rows: torch.Tensor
+    factor: float = 1.0
+
+
+@dataclass
+class RowVector:
+    """One vector (float32 [d]) that is added to every row of the residual stream."""
+    vector: torch.Tensor
+
+
 class Residual:
-    """The float32 residual stream [T, d] plus the branch outputs not yet added to it (tensors, or
-    ``ScaledBranch``es).  The next norm adds them and normalizes in one kernel.
+    """The float32 residual stream [T, d] plus the branch outputs not yet added to it (tensors,
+    ``ScaledBranch``es, ``WeightedBranch``es or ``RowVector``s).  The next norm adds them and normalizes in one kernel.
 
     ``next_norm``: (weight, eps) of the norm that the layer after the one running starts with (the final norm
     after the last), if that norm is a root-mean-square norm, set by whoever runs the layers; a layer whose last

@@ -6,7 +6,7 @@ from typing import Dict
 import torch
 
 from ..weights.loader import Expect
-from .base import BuildContext, Residual, ScaledBranch, part_class
+from .base import BuildContext, Residual, ScaledBranch, WeightedBranch, part_class
 
 _ARRANGEMENTS: Dict[str, type] = {}
 _FUSIONS: Dict[str, object] = {}
@@ -68,8 +68,8 @@ class ParallelPreNormBlock:
     All mixers read the same normed input and their outputs are summed into the residual
     (reference: src/decoder.rs:2658-2682, 2684-2699).  With one mixer this is the ordinary
     sequential pre-norm layer.  A layer may scale either branch feature by feature before the add
-    (``mixer_scale_name`` / ``ffn_scale_name``: h += scale * branch, the product in float32), and may have no
-    feed-forward at all (``ffn`` None)."""
+    (``mixer_scale_name`` / ``ffn_scale_name``: h += scale * branch, the product in float32) or multiply both by
+    one number (``branch_multiplier``), and may have no feed-forward at all (``ffn`` None)."""
 
     @classmethod
     def expected_tensors(cls, layer, hidden_size: int):
@@ -131,7 +131,9 @@ class ParallelPreNormBlock:
         self.ffn_scale = scale(layer.ffn_scale_name) if layer.ffn is not None else None
         factory = _FUSIONS.get(layer.arrangement)
         # the fast path knows plain branches and a feed-forward behind them; None when parts or sizes do not fit
-        plain = self.mixer_scale is None and self.ffn_scale is None and self.ffn is not None
+        self.branch_multiplier = float(getattr(layer, "branch_multiplier", 1.0))
+        plain = (self.mixer_scale is None and self.ffn_scale is None and self.ffn is not None
+                 and self.branch_multiplier == 1.0)
         self.fusion = factory(self, build) if factory is not None and plain else None
 
     @property
@@ -174,9 +176,16 @@ class ParallelPreNormBlock:
             outputs = [mixer.forward(normed, step, caches[name]) for name, mixer in self.mixers]
         if self.mixer_scale is not None:
             outputs = [ScaledBranch(rows, self.mixer_scale) for rows in outputs]
+        elif self.branch_multiplier != 1.0:
+            outputs = [WeightedBranch(rows, self.branch_multiplier) for rows in outputs]
         residual.pending = outputs
         if self.ffn is None:
             return
         normed = self.ffn_norm.forward(residual)
         rows = self.ffn.forward(normed)
-        residual.pending = [rows if self.ffn_scale is None else ScaledBranch(rows, self.ffn_scale)]
+        if self.ffn_scale is not None:
+            residual.pending = [ScaledBranch(rows, self.ffn_scale)]
+        elif self.branch_multiplier != 1.0:
+            residual.pending = [WeightedBranch(rows, self.branch_multiplier)]
+        else:
+            residual.pending = [rows]

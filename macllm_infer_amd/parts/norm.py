@@ -1,4 +1,4 @@
-"""RMSNorm fused with the residual add that precedes it."""
+"""Norms fused with the residual add that precedes them."""
 from __future__ import annotations
 
 from typing import Optional
@@ -8,7 +8,7 @@ import torch
 from ..kernels import ops
 from ..kernels.limits import NORM_MAX_WIDTH, beyond
 from ..weights.loader import Expect
-from .base import BuildContext, Part, Residual, ScaledBranch, register_part
+from .base import BuildContext, Part, Residual, RowVector, ScaledBranch, WeightedBranch, register_part
 
 
 def partial_slab(pending) -> Optional[torch.Tensor]:
@@ -24,6 +24,21 @@ def partial_slab(pending) -> Optional[torch.Tensor]:
         if slab._base is not base or slab.shape != base.shape[1:] or slab.data_ptr() != base[index].data_ptr():
             return None
     return base
+
+
+def fold_weighted(residual: Residual) -> None:
+    """Add the ``WeightedBranch``es and ``RowVector``s among the pending branches to the stream with the kernel
+    that knows them, and leave the others pending: for a norm whose own kernel fuses neither."""
+    kept = []
+    for branch in residual.pending:
+        if isinstance(branch, WeightedBranch):
+            ops.stream_add(residual.h, branch.rows, branch.factor, None)
+        elif isinstance(branch, RowVector):
+            ops.stream_add(residual.h, None, 1.0, branch.vector)
+        else:
+            kept.append(branch)
+    if len(kept) != len(residual.pending):
+        residual.pending = kept
 
 
 @register_part("rmsnorm")
@@ -59,6 +74,8 @@ class RmsNorm(Part):
     def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add the pending branch outputs to the residual stream and return its normed rows
         (all of them, or only ``rows``; with ``rows`` the stream itself is left unchanged)."""
+        if any(isinstance(branch, (WeightedBranch, RowVector)) for branch in residual.pending):
+            fold_weighted(residual)
         pending = residual.pending
         slab = partial_slab(pending)
         if slab is not None and slab.shape[0] <= 16 and residual.h.shape[1] % 4 == 0:
@@ -93,4 +110,61 @@ class RmsNorm(Part):
         ops.add_rmsnorm(residual.h, pending, self.weight, self.eps, out, rows)
         if rows is None:
             residual.pending = []
+        return out
+
+
+LAYERNORM_BRANCHES = 3          # branches that the layer norm's kernel adds in its own launch
+
+
+@register_part("layernorm")
+class LayerNorm(Part):
+    """y = (x - mean) / sqrt(variance + eps) * weight + bias over a row, mean and variance (the mean of the squared
+    deviations, taken in a second pass over the row) in float32.  The kernel first adds what is pending to the
+    stream: up to three branches, each times a number of its own, and one vector for every row."""
+    graph_safe = True
+    kernel_modules = ("common",)
+
+    @classmethod
+    def expected_tensors(cls, spec, prefix: str, hidden_size: int):
+        return [Expect(f"{prefix}.weight", ((hidden_size,),), init="norm"),
+                Expect(f"{prefix}.bias", ((hidden_size,),), init="bias")]
+
+    @classmethod
+    def limits(cls, spec, hidden_size: int):
+        return beyond("layernorm", "hidden_size", hidden_size, NORM_MAX_WIDTH, "the norm stages a float32 row in 64 KiB of LDS")
+
+    def __init__(self, spec, prefix: str, tensors, build: BuildContext):
+        self.eps = spec.eps
+        self.build = build
+        self.weight = tensors[f"{prefix}.weight"].to(torch.float32).contiguous().to(build.device)
+        self.bias = tensors[f"{prefix}.bias"].to(torch.float32).contiguous().to(build.device)
+
+    def forward(self, residual: Residual, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Add the pending branches to the stream and return its normed rows (all, or only ``rows``; with ``rows``
+        the stream itself is left unchanged and the branches stay pending)."""
+        branches, vector = [], None
+        for branch in residual.pending:
+            if isinstance(branch, RowVector):
+                if vector is None:
+                    vector = branch.vector
+                else:                                      # a second vector: added by the plain kernel
+                    ops.stream_add(residual.h, None, 1.0, branch.vector)
+            elif isinstance(branch, ScaledBranch):         # a scale by feature: the kernel that knows it adds it
+                ops.add_scaled_rmsnorm(residual.h, branch.rows, branch.scale, self.weight, self.eps, None)
+            elif isinstance(branch, WeightedBranch):
+                branches.append((branch.rows, float(branch.factor)))
+            else:
+                branches.append((branch, 1.0))
+        while len(branches) > LAYERNORM_BRANCHES:
+            first, factor = branches.pop(0)
+            ops.stream_add(residual.h, first, factor, None)
+        count = residual.h.shape[0] if rows is None else rows.numel()
+        out = torch.empty((count, residual.h.shape[1]), dtype=self.build.dtype, device=residual.h.device)
+        ops.add_layernorm(residual.h, branches, vector, self.weight, self.bias, self.eps, out, rows)
+        if rows is None:
+            residual.pending = []
+        else:
+            # the stream was not changed: what this call could not fuse was added above, the rest stays pending
+            kept = [WeightedBranch(tensor, factor) for tensor, factor in branches]
+            residual.pending = kept + ([RowVector(vector)] if vector is not None else [])
         return out

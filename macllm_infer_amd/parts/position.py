@@ -34,6 +34,13 @@ class PositionEncoding(Part):
         layer then runs this part's own ``rotate_and_store`` and the general kernels."""
         return None
 
+    def pair_rotation(self):
+        """``(inv_freq or None, rotary_dim, interleaved)`` of an encoding that turns pairs of dimensions by
+        position * inv_freq[i]: pair i is dimensions (i, i + rotary_dim / 2) (half-split) or (2i, 2i + 1)
+        (``interleaved``); ``(None, 0, False)``: nothing is turned.  None: the encoding is no such rotation.  For
+        mixers whose kernels turn a part of their rows themselves."""
+        return None
+
     def rotate(self, qkv, num_heads, num_kv_heads, head_dim, step) -> None:
         return None
 
@@ -54,6 +61,9 @@ class NoPosition(PositionEncoding):
     def fused_rotation(self):
         return None, 0
 
+    def pair_rotation(self):
+        return None, 0, False
+
 
 @register_part("rope")
 class Rope(PositionEncoding):
@@ -69,6 +79,9 @@ class Rope(PositionEncoding):
 
     def fused_rotation(self):
         return self.inv_freq, self.rotary_dim
+
+    def pair_rotation(self):
+        return self.inv_freq, self.rotary_dim, False
 
     def rotate_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step, cache) -> None:
         owns = cache.owns_kv
@@ -95,3 +108,20 @@ class LogDistanceBias(PositionEncoding):
 
     def fused_rotation(self):
         return None
+
+
+@register_part("rope_interleaved")
+class InterleavedRope(PositionEncoding):
+    """Rotary encoding whose pairs are neighbouring dimensions: (u, v) = dimensions (2i, 2i + 1) at position p
+    become (u cos a - v sin a, v cos a + u sin a), a = p * theta^(-2i / rotary_dim); frequencies formed in float64
+    and rounded to float32, angles, cos and sin in float32.  The mixers that use it turn their rows in kernels of
+    their own (``pair_rotation``)."""
+    graph_safe = True
+
+    def __init__(self, spec, head_dim: int, build: BuildContext):
+        self.rotary_dim = spec.rotary_dim
+        frequencies = [spec.theta ** (-index / spec.rotary_dim) for index in range(0, spec.rotary_dim, 2)]
+        self.inv_freq = torch.tensor(frequencies, dtype=torch.float64).to(torch.float32).to(build.device)
+
+    def pair_rotation(self):
+        return self.inv_freq, self.rotary_dim, True

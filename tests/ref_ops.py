@@ -299,9 +299,183 @@ def argmax(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
+# --------------------------------------------------------------------------- bigram embedding, layer norm
+def embed_bigram(token_ids, table, multiplier, bigram, buckets, mul_prev, mul_cur, positions, lane_of_token,
+                 cu_seqlens, slot_ids, previous, out):
+    """out[t] = table[token] * multiplier + bigram[row], row = (token before * mul_prev + token * mul_cur) mod
+    buckets, the last row (``buckets``) at position 0; the token before a lane's first one is
+    ``previous[slot of the lane]``, which then takes the lane's last token."""
+    ids = token_ids.long()
+    rows = torch.empty_like(ids)
+    for token in range(ids.numel()):
+        lane = int(lane_of_token[token])
+        if int(positions[token]) == 0:
+            rows[token] = buckets
+            continue
+        before = int(previous[int(slot_ids[lane]), 0]) if token == int(cu_seqlens[lane]) else int(ids[token - 1])
+        rows[token] = (before * mul_prev + int(ids[token]) * mul_cur) % buckets
+    out.copy_(_f(table)[ids] * multiplier + _f(bigram)[rows])
+    for lane in range(slot_ids.numel()):
+        if int(cu_seqlens[lane + 1]) > int(cu_seqlens[lane]):
+            previous[int(slot_ids[lane]), 0] = token_ids[int(cu_seqlens[lane + 1]) - 1]
+
+
+def stream_add(h, rows, factor, vector):
+    if rows is not None:
+        h += float(factor) * _f(rows)
+    if vector is not None:
+        h += vector
+
+
+def add_layernorm(h, branches, vector, weight, bias, eps, out, rows=None):
+    total = h.clone()
+    for tensor, factor in branches:
+        total = total + float(factor) * _f(tensor)
+    if vector is not None:
+        total = total + vector
+    if rows is None:
+        h.copy_(total)
+        picked = total
+    else:
+        picked = total[rows.long()]
+    if out is not None:
+        mean = picked.mean(dim=-1, keepdim=True)
+        centred = picked - mean
+        variance = (centred * centred).mean(dim=-1, keepdim=True)
+        out.copy_((centred / torch.sqrt(variance + eps) * weight + bias).to(out.dtype))
+
+
+def clamped_glu(gate_up, limit, alpha, up_offset, out):
+    inner = out.shape[1]
+    gate = _f(gate_up[:, :inner]).clamp(max=limit)
+    up = _f(gate_up[:, inner:2 * inner]).clamp(min=-limit, max=limit)
+    out.copy_((gate * torch.sigmoid(alpha * gate) * (up + up_offset)).to(out.dtype))
+
+
+# --------------------------------------------------------------------------- latent attention
+def _turn(x, positions, inv_freq, rotary_dim, interleaved):
+    """x float32 [T, ..., width]: its first ``rotary_dim`` dimensions turned in pairs."""
+    if inv_freq is None or rotary_dim == 0:
+        return x
+    half = rotary_dim // 2
+    angle = positions.to(torch.float32).reshape(-1, *([1] * (x.dim() - 1))) * inv_freq
+    cos, sin = angle.cos(), angle.sin()
+    out = x.clone()
+    if interleaved:
+        a, b = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+        out[..., 0:rotary_dim:2] = a * cos - b * sin
+        out[..., 1:rotary_dim:2] = b * cos + a * sin
+    else:
+        a, b = x[..., :half], x[..., half:rotary_dim]
+        out[..., :half] = a * cos - b * sin
+        out[..., half:rotary_dim] = b * cos + a * sin
+    return out
+
+
+def latent_prepare(down, q_rank, kv_rank, rope_dim, q_norm, kv_norm, eps, positions, inv_freq, rotary_dim,
+                   interleaved, slot_mapping, k_cache, v_cache, query_latent):
+    rows = _f(down)
+    def rms(x, weight):
+        return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * weight
+    query_latent.copy_(rms(rows[:, :q_rank], q_norm).to(query_latent.dtype))
+    if slot_mapping is None:
+        return
+    latent = rms(rows[:, q_rank:q_rank + kv_rank], kv_norm)
+    turned = _turn(rows[:, q_rank + kv_rank:q_rank + kv_rank + rope_dim], positions, inv_freq, rotary_dim, interleaved)
+    page_size = k_cache.shape[2]
+    pages = (slot_mapping // page_size).long()
+    offsets = (slot_mapping % page_size).long()
+    k_cache[pages, 0, offsets, :] = torch.cat([latent, turned], dim=1).to(k_cache.dtype)
+    v_cache[pages, 0, :, offsets] = latent.to(v_cache.dtype)
+
+
+def head_linear(x, x_col, x_head_stride, weight, out, out_col, out_head_stride):
+    heads, features, inner = weight.shape
+    for head in range(heads):
+        rows = _f(x[:, x_col + head * x_head_stride:x_col + head * x_head_stride + inner])
+        first = out_col + head * out_head_stride
+        out[:, first:first + features] = (rows @ _f(weight[head]).T).to(out.dtype)
+
+
+def rotate_heads(x, col, head_stride, num_heads, width, positions, inv_freq, rotary_dim, interleaved, out, out_col,
+                 out_head_stride):
+    for head in range(num_heads):
+        rows = _f(x[:, col + head * head_stride:col + head * head_stride + width])
+        first = out_col + head * out_head_stride
+        out[:, first:first + width] = _turn(rows, positions, inv_freq, rotary_dim, interleaved).to(out.dtype)
+
+
+def latent_attention_supported(dtype, num_heads, kv_rank, rope_dim, page_size):
+    return False
+
+
+# --------------------------------------------------------------------------- routed experts
+def moe_route(logits, num_experts, top_k, correction, scale, eps, shared_gate):
+    scores = torch.softmax(_f(logits[:, :num_experts]), dim=-1)
+    chosen = torch.topk(scores + correction, top_k, dim=-1).indices
+    picked = torch.gather(scores, 1, chosen)
+    weights = picked / (picked.sum(dim=-1, keepdim=True) + eps) * scale
+    gate = torch.sigmoid(_f(logits[:, num_experts])) if shared_gate else None
+    return chosen.to(torch.int32), weights, gate
+
+
+class MoePlan:
+    def __init__(self, chosen, num_experts, pad=16):
+        tokens, top_k = chosen.shape
+        self.pad, self.tokens, self.top_k = pad, tokens, top_k
+        self.capacity = -(-(tokens * top_k + num_experts * (pad - 1)) // pad) * pad
+        self.source = torch.full((self.capacity,), -1, dtype=torch.int32)
+        self.place = torch.zeros((tokens * top_k,), dtype=torch.int32)
+        self.tile_expert = torch.full((self.capacity // pad,), -1, dtype=torch.int32)
+        cursor = 0
+        flat = chosen.reshape(-1)
+        for expert in range(num_experts):
+            entries = torch.nonzero(flat == expert).reshape(-1)
+            for index, entry in enumerate(entries.tolist()):
+                self.source[cursor + index] = entry // top_k
+                self.place[entry] = cursor + index
+            tiles = -(-len(entries) // pad)
+            self.tile_expert[cursor // pad:cursor // pad + tiles] = expert
+            cursor += tiles * pad
+
+
+def moe_plan(chosen, num_experts):
+    return MoePlan(chosen, num_experts)
+
+
+def moe_expert_gemm(x, plan, weight, out, gather, glu):
+    out.zero_()
+    for tile in range(plan.tile_expert.numel()):
+        expert = int(plan.tile_expert[tile])
+        if expert < 0:
+            continue
+        for place in range(tile * plan.pad, (tile + 1) * plan.pad):
+            source = int(plan.source[place])
+            if source < 0:
+                continue
+            row = _f(x[source if gather else place])
+            sums = _f(weight[expert]) @ row
+            if glu is not None:
+                inner = sums.numel() // 2
+                gate = sums[:inner].clamp(max=glu.limit)
+                up = sums[inner:].clamp(min=-glu.limit, max=glu.limit)
+                sums = gate * torch.sigmoid(glu.alpha * gate) * (up + glu.up_offset)
+            out[place] = sums.to(out.dtype)
+
+
+def moe_combine(down, plan, weights, shared_rows, shared_gate, out):
+    places = plan.place.long().reshape(plan.tokens, plan.top_k)
+    total = (down[places] * weights[:, :, None]).sum(dim=1)
+    if shared_rows is not None:
+        total = total + shared_gate[:, None] * _f(shared_rows)
+    out.copy_(total)
+
+
 NAMES = ["fused_gemm_split", "add_partials_rmsnorm", "prefill_attention_supported", "decode_attention_supported", "decode_attention", "embed", "add_rmsnorm", "swiglu", "scale_to_f32", "tanh_softcap", "linear", "rope_kv_store", "paged_attention",
          "conv1d_silu", "conv_state_update", "conv_step", "ssm_scan", "gate_norm", "argmax", "feed_tokens", "keep_allowed",
-         "add_scaled_rmsnorm", "polynorm", "tanh_rows", "head_norm_gate", "linear_state_scan"]
+         "add_scaled_rmsnorm", "polynorm", "tanh_rows", "head_norm_gate", "linear_state_scan",
+         "embed_bigram", "stream_add", "add_layernorm", "clamped_glu", "latent_prepare", "head_linear", "rotate_heads",
+         "latent_attention_supported", "moe_route", "moe_plan", "moe_expert_gemm", "moe_combine"]
 
 
 def install(monkeypatch):
