@@ -506,3 +506,192 @@ extern "C" int mi_polynorm(const void* z, int dtype, long ld, const float* coeff
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
+
+// ---------------------------------------------------------------- embedding with a hashed bigram row
+// h[t, :] = table[ids[t], :] * multiplier + bigram[row, :], row = (token before * mul_prev + token * mul_cur) mod
+// buckets, or `buckets` (the table's last row) for the token at position 0.  The token before a lane's first
+// one is the request's state, previous[slot]; a second, tiny launch leaves the lane's last token there (a launch
+// of its own: the rows of a lane are read by many workgroups).
+template <typename T>
+__global__ void embed_bigram_kernel(const int* __restrict__ ids, const T* __restrict__ table, float multiplier,
+                                    const T* __restrict__ bigram, int buckets, long mul_prev, long mul_cur,
+                                    const int* __restrict__ positions, const int* __restrict__ lane_of_token,
+                                    const int* __restrict__ cu_seqlens, const int* __restrict__ slot_ids,
+                                    const int* __restrict__ previous, float* __restrict__ h, int d) {
+  const long token = blockIdx.x;
+  const int id = ids[token];
+  long row = buckets;
+  if (positions[token] != 0) {
+    const int lane = lane_of_token[token];
+    const long before = token == cu_seqlens[lane] ? previous[slot_ids[lane]] : ids[token - 1];
+    row = (before * mul_prev + (long)id * mul_cur) % buckets;
+    if (row < 0) row += buckets;
+  }
+  const T* first = table + (long)id * d;
+  const T* second = bigram + row * d;
+  float* out = h + token * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) out[i] = fmaf(to_float(first[i]), multiplier, to_float(second[i]));
+}
+
+__global__ void keep_last_token_kernel(const int* __restrict__ ids, const int* __restrict__ cu_seqlens,
+                                       const int* __restrict__ slot_ids, int* __restrict__ previous, int lanes) {
+  const int lane = blockIdx.x * blockDim.x + threadIdx.x;
+  if (lane >= lanes) return;
+  const int end = cu_seqlens[lane + 1];
+  if (end > cu_seqlens[lane]) previous[slot_ids[lane]] = ids[end - 1];
+}
+
+extern "C" int mi_embed_bigram(const int* ids, const void* table, int table_dtype, float multiplier, const void* bigram,
+                               int buckets, long mul_prev, long mul_cur, const int* positions, const int* lane_of_token,
+                               const int* cu_seqlens, const int* slot_ids, int* previous, float* h, int T, int d,
+                               int lanes, hipStream_t stream) {
+  if (T <= 0 || d <= 0 || lanes <= 0 || buckets <= 0 || !ids || !table || !bigram || !positions || !lane_of_token ||
+      !cu_seqlens || !slot_ids || !previous || !h)
+    return ERR_BAD_ARGUMENT;
+  if (table_dtype == DT_F32)
+    embed_bigram_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, multiplier, (const float*)bigram, buckets,
+                                                      mul_prev, mul_cur, positions, lane_of_token, cu_seqlens, slot_ids,
+                                                      previous, h, d);
+  else if (table_dtype == DT_BF16)
+    embed_bigram_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, (const bf16_t*)table, multiplier, (const bf16_t*)bigram,
+                                                       buckets, mul_prev, mul_cur, positions, lane_of_token, cu_seqlens,
+                                                       slot_ids, previous, h, d);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  keep_last_token_kernel<<<(lanes + 255) / 256, 256, 0, stream>>>(ids, cu_seqlens, slot_ids, previous, lanes);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- h += factor * rows + vector
+template <typename T>
+__global__ void stream_add_kernel(float* __restrict__ h, const T* __restrict__ rows, float factor,
+                                  const float* __restrict__ vector, long total, int d) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float value = h[i];
+  if (rows) value = fmaf(factor, to_float(rows[i]), value);
+  if (vector) value += vector[i % d];
+  h[i] = value;
+}
+
+extern "C" int mi_stream_add(float* h, const void* rows, int rows_dtype, float factor, const float* vector, int T, int d,
+                             hipStream_t stream) {
+  if (!h || T <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  const long total = (long)T * d;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (rows_dtype == DT_F32)
+    stream_add_kernel<float><<<blocks, 256, 0, stream>>>(h, (const float*)rows, factor, vector, total, d);
+  else if (rows_dtype == DT_BF16)
+    stream_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)rows, factor, vector, total, d);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- residual add + layer norm
+// v = h + f0 b0 + f1 b1 + f2 b2 + vector (float32; written back to h unless rows are gathered);
+// out = (v - mean) / sqrt(mean((v - mean)^2) + eps) * weight + bias.  The row is kept in LDS; the variance is
+// taken from the deviations in a second pass over it.  One workgroup a row.
+struct NormBranch {
+  const void* rows;
+  int dtype;
+  float factor;
+};
+
+__device__ __forceinline__ float branch_value(const NormBranch& branch, long at) {
+  if (!branch.rows) return 0.f;
+  const float value = branch.dtype == DT_BF16 ? (float)((const bf16_t*)branch.rows)[at] : ((const float*)branch.rows)[at];
+  return branch.factor * value;
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(1024)
+add_layernorm_kernel(float* __restrict__ h, NormBranch b0, NormBranch b1, NormBranch b2, const float* __restrict__ vector,
+                     const float* __restrict__ weight, const float* __restrict__ bias, float eps, TO* __restrict__ out,
+                     const int* __restrict__ rows, int d) {
+  extern __shared__ float wide_row[];
+  __shared__ float scratch[16];
+  const long out_row = blockIdx.x;
+  const long row = rows ? (long)rows[out_row] : out_row;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const long at = row * d + i;
+    float v = h[at];
+    v += branch_value(b0, at);
+    v += branch_value(b1, at);
+    v += branch_value(b2, at);
+    if (vector) v += vector[i];
+    if (!rows) h[at] = v;
+    wide_row[i] = v;
+    sum += v;
+  }
+  if (!out) return;
+  const float mean = block_sum(sum, scratch) / (float)d;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const float centred = wide_row[i] - mean;
+    squares += centred * centred;
+  }
+  const float variance = block_sum(squares, scratch) / (float)d;
+  const float denominator = sqrtf(variance + eps);
+  TO* o = out + out_row * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x)
+    o[i] = from_float<TO>((wide_row[i] - mean) / denominator * weight[i] + bias[i]);
+}
+
+extern "C" int mi_add_layernorm(float* h, const void* rows0, int dtype0, float factor0, const void* rows1, int dtype1,
+                                float factor1, const void* rows2, int dtype2, float factor2, const float* vector,
+                                const float* weight, const float* bias, float eps, void* out, int out_dtype,
+                                const int* rows, int n_rows, int d, hipStream_t stream) {
+  if (!h || !weight || !bias || n_rows <= 0 || d <= 0) return ERR_BAD_ARGUMENT;
+  if ((size_t)d * sizeof(float) > 64 * 1024) return ERR_UNSUPPORTED_SIZE;
+  const NormBranch b0 = {rows0, dtype0, factor0}, b1 = {rows1, dtype1, factor1}, b2 = {rows2, dtype2, factor2};
+  const int threads = (d > 2048 && n_rows <= 512) ? 1024 : 256;
+  const size_t lds = (size_t)d * sizeof(float);
+  if (out_dtype == DT_F32)
+    add_layernorm_kernel<float><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, (float*)out, rows, d);
+  else if (out_dtype == DT_BF16)
+    add_layernorm_kernel<bf16_t><<<n_rows, threads, lds, stream>>>(h, b0, b1, b2, vector, weight, bias, eps, (bf16_t*)out, rows, d);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- clamped gated activation
+// out[t, i] = g * sigmoid(alpha g) * (u + offset), g = min(gate, limit), u = clamp(up, -limit, limit); a row of
+// gate_up holds [gate | up].
+__device__ __forceinline__ float clamped_glu_f(float gate, float up, float limit, float alpha, float offset) {
+  const float g = fminf(gate, limit);
+  const float u = fminf(fmaxf(up, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + offset);
+}
+
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gate_up, long ld, T* __restrict__ out, long out_ld, int I,
+                                   long total, float limit, float alpha, float offset) {
+  const long at = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (at >= total) return;
+  const long t = at / I;
+  const int i = (int)(at % I);
+  const T* row = gate_up + t * ld;
+  out[t * out_ld + i] = from_float<T>(clamped_glu_f(to_float(row[i]), to_float(row[I + i]), limit, alpha, offset));
+}
+
+extern "C" int mi_clamped_glu(const void* gate_up, int dtype, long ld, void* out, long out_ld, int T, int I, float limit,
+                              float alpha, float offset, hipStream_t stream) {
+  if (!gate_up || !out || T <= 0 || I <= 0 || ld < 2L * I || out_ld < I) return ERR_BAD_ARGUMENT;
+  const long total = (long)T * I;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == DT_F32)
+    clamped_glu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, ld, (float*)out, out_ld, I, total, limit, alpha, offset);
+  else if (dtype == DT_BF16)
+    clamped_glu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gate_up, ld, (bf16_t*)out, out_ld, I, total, limit, alpha, offset);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

@@ -1,0 +1,270 @@
+// A feed-forward of many small experts of which a token uses a few.
+//
+//   moe_route        float32 router logits -> softmax, correction, the token's experts and their weights (one wave
+//                    a token), and the sigmoid of the shared expert's gate logit
+//   moe_plan         the step's (token, choice) rows grouped by expert, every expert's rows starting a tile of 16
+//                    places: built on the device by one workgroup, so that no count has to travel to the host and
+//                    the launches that follow depend on the number of tokens alone
+//   moe_expert_gemm  the grouped product on the matrix cores: a tile's rows (gathered from the tokens' rows, or
+//                    the places themselves) with its expert's matrix; epilogue: plain, or the clamped gated
+//                    activation of a gate tile and an up tile
+//   moe_combine      a token's weighted sum over its choices, in their order, plus the gated shared expert
+//
+// A row of a tile is summed on its own (a column of the matrix cores' result), so a token's numbers do not depend
+// on which other rows share its tile or on the place it was given.
+#include "mfma_tile.h"
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_PER_LANE (MOE_MAX_EXPERTS / WAVE)
+
+// ---------------------------------------------------------------- router
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int top, const float* __restrict__ correction,
+                 float scale, float eps, int* __restrict__ chosen, float* __restrict__ weights, float* __restrict__ gate) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int token = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (token >= T) return;
+  const float* row = logits + (long)token * ld;
+  float score[MOE_PER_LANE], choice[MOE_PER_LANE];
+  float most = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < MOE_PER_LANE; ++j) {
+    const int e = lane + WAVE * j;
+    score[j] = e < E ? row[e] : -INFINITY;
+    most = fmaxf(most, score[j]);
+  }
+  most = wave_max(most);
+  float total = 0.f;
+#pragma unroll
+  for (int j = 0; j < MOE_PER_LANE; ++j) {
+    const int e = lane + WAVE * j;
+    score[j] = e < E ? expf(score[j] - most) : 0.f;
+    total += score[j];
+  }
+  total = wave_sum(total);
+#pragma unroll
+  for (int j = 0; j < MOE_PER_LANE; ++j) {
+    const int e = lane + WAVE * j;
+    score[j] = score[j] / total;
+    choice[j] = e < E ? score[j] + correction[e] : -INFINITY;
+  }
+  float picked_sum = 0.f;
+  float mine = 0.f;            // lane k keeps the score of the k-th choice
+  int mine_id = 0;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY, best_score = 0.f;
+    int best_id = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      const int e = lane + WAVE * j;
+      if (e < E && (choice[j] > best || (choice[j] == best && e < best_id))) {
+        best = choice[j];
+        best_id = e;
+        best_score = score[j];
+      }
+    }
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, WAVE);
+      const int other_id = __shfl_xor(best_id, offset, WAVE);
+      const float other_score = __shfl_xor(best_score, offset, WAVE);
+      if (other > best || (other == best && other_id < best_id)) {
+        best = other;
+        best_id = other_id;
+        best_score = other_score;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j)
+      if (lane + WAVE * j == best_id) choice[j] = -INFINITY;
+    picked_sum += best_score;
+    if ((k & (WAVE - 1)) == lane) {
+      // more choices than lanes: written as they come
+      mine = best_score;
+      mine_id = best_id;
+    }
+    if (top > WAVE && lane == 0) {
+      chosen[(long)token * top + k] = best_id;
+      weights[(long)token * top + k] = best_score;      // divided below
+    }
+  }
+  const float denominator = picked_sum + eps;
+  if (top <= WAVE) {
+    if (lane < top) {
+      chosen[(long)token * top + lane] = mine_id;
+      weights[(long)token * top + lane] = mine / denominator * scale;
+    }
+  } else if (lane == 0) {
+    for (int k = 0; k < top; ++k) weights[(long)token * top + k] = weights[(long)token * top + k] / denominator * scale;
+  }
+  if (gate && lane == 0) gate[token] = 1.0f / (1.0f + expf(-row[E]));
+}
+
+extern "C" int mi_moe_route(const float* logits, long ld, int T, int E, int top, const float* correction, float scale,
+                            float eps, int* chosen, float* weights, float* gate, hipStream_t stream) {
+  if (!logits || !correction || !chosen || !weights || T <= 0 || E <= 0 || top <= 0 || top > E || ld < E + (gate ? 1 : 0))
+    return ERR_BAD_ARGUMENT;
+  if (E > MOE_MAX_EXPERTS) return ERR_UNSUPPORTED_SIZE;
+  moe_route_kernel<<<(T + 3) / 4, 256, 0, stream>>>(logits, ld, T, E, top, correction, scale, eps, chosen, weights, gate);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- rows grouped by expert
+__global__ void __launch_bounds__(1024)
+moe_plan_kernel(const int* __restrict__ chosen, int entries, int top, int E, int pad, int capacity,
+                int* __restrict__ source, int* __restrict__ place, int* __restrict__ tile_expert, int* __restrict__ ranks) {
+  __shared__ int counts[MOE_MAX_EXPERTS];
+  __shared__ int offsets[MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  const int threads = blockDim.x;
+  for (int e = tid; e < E; e += threads) counts[e] = 0;
+  for (int i = tid; i < capacity; i += threads) source[i] = -1;
+  for (int t = tid; t < capacity / pad; t += threads) tile_expert[t] = -1;
+  __syncthreads();
+  for (int i = tid; i < entries; i += threads) ranks[i] = atomicAdd(&counts[chosen[i]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int running = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = running;
+      running += (counts[e] + pad - 1) / pad * pad;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += threads) {
+    const int first = offsets[e] / pad;
+    const int tiles = (counts[e] + pad - 1) / pad;
+    for (int t = 0; t < tiles; ++t) tile_expert[first + t] = e;
+  }
+  for (int i = tid; i < entries; i += threads) {
+    const int at = offsets[chosen[i]] + ranks[i];
+    source[at] = i / top;
+    place[i] = at;
+  }
+}
+
+extern "C" int mi_moe_plan(const int* chosen, int entries, int top, int E, int pad, int capacity, int* source, int* place,
+                           int* tile_expert, int* ranks, hipStream_t stream) {
+  if (!chosen || !source || !place || !tile_expert || !ranks || entries <= 0 || top <= 0 || E <= 0 || pad <= 0 ||
+      capacity % pad != 0 || capacity < entries + E * (pad - 1))
+    return ERR_BAD_ARGUMENT;
+  if (E > MOE_MAX_EXPERTS) return ERR_UNSUPPORTED_SIZE;
+  moe_plan_kernel<<<1, 1024, 0, stream>>>(chosen, entries, top, E, pad, capacity, source, place, tile_expert, ranks);
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- the grouped product
+// Tile t of 16 places belongs to expert tile_expert[t] (none: the workgroup leaves).  GLU: the expert's matrix is
+// [2 I, K], gate rows then up rows; out[place, n] = act(gate tile, up tile), n < I.  Places without a row get zeros.
+template <typename T, typename TO, bool VEC, bool GLU>
+__global__ void __launch_bounds__(TILE_THREADS)
+moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride, long ldw,
+                       int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert, int gather,
+                       float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+  __shared__ float red[TILE_WAVES][256];
+  const int tile = blockIdx.y;
+  const int expert = tile_expert[tile];
+  if (expert < 0) return;
+  const int tid = threadIdx.x;
+  const int r = (tid & (WAVE - 1)) % 16;
+  const int width = GLU ? N / 2 : N;
+  const long n0 = (long)blockIdx.x * 16;
+  const T* matrix = W + (long)expert * expert_stride;
+  const long n_row = min(n0 + r, (long)width - 1);
+  const int place_in = tile * 16 + r;
+  const int from = source[place_in];
+  const long x_at = gather ? max(from, 0) : place_in;
+  const T* x_row[1] = {x + min(x_at, (long)x_rows - 1) * ldx};
+  constexpr int NT = GLU ? 2 : 1;
+  const T* w_row[NT];
+  w_row[0] = matrix + n_row * ldw;
+  if (GLU) w_row[NT - 1] = matrix + (width + n_row) * ldw;
+  tile_floatx4 acc[NT][1];
+  tile_accumulate<T, 1, NT, VEC>(w_row, x_row, K, acc);
+  float value = tile_reduce(acc[0][0], red);
+  if (GLU) {
+    const float up = tile_reduce(acc[NT - 1][0], red);
+    const float g = fminf(value, limit);
+    const float u = fminf(fmaxf(up, -limit), limit);
+    value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+  }
+  const int l = tid % 64;
+  const long n = n0 + 4 * (l / 16) + tid / 64;
+  const int place = tile * 16 + (l % 16);
+  if (n < width) out[(long)place * ldo + n] = from_float<TO>(source[place] >= 0 ? value : 0.f);
+}
+
+template <typename T, typename TO>
+static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, long expert_stride, long ldw, int N, int K,
+                               const int* source, const int* tile_expert, int tiles, int gather, int glu, float limit,
+                               float alpha, float offset, TO* out, long ldo, hipStream_t stream) {
+  constexpr int PIECE = TileTraits<T>::PIECE;
+  const bool vec = K % PIECE == 0 && ldx % PIECE == 0 && ldw % PIECE == 0 && expert_stride % PIECE == 0 &&
+                   ((unsigned long long)x % 16) == 0 && ((unsigned long long)W % 16) == 0;
+  const int width = glu ? N / 2 : N;
+  const dim3 grid((unsigned)((width + 15) / 16), (unsigned)tiles);
+#define EXPERT_LAUNCH(VEC_, GLU_)                                                                                      \
+  moe_expert_gemm_kernel<T, TO, VEC_, GLU_><<<grid, TILE_THREADS, 0, stream>>>(                                       \
+      x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
+  if (vec && glu) EXPERT_LAUNCH(true, true);
+  else if (vec) EXPERT_LAUNCH(true, false);
+  else if (glu) EXPERT_LAUNCH(false, true);
+  else EXPERT_LAUNCH(false, false);
+#undef EXPERT_LAUNCH
+}
+
+extern "C" int mi_moe_expert_gemm(const void* x, int dtype, long ldx, int x_rows, const void* W, long expert_stride,
+                                  long ldw, int N, int K, const int* source, const int* tile_expert, int tiles, int pad,
+                                  int gather, int glu, float limit, float alpha, float offset, void* out, int out_dtype,
+                                  long ldo, hipStream_t stream) {
+  if (!x || !W || !source || !tile_expert || !out || x_rows <= 0 || N <= 0 || K <= 0 || tiles <= 0 || ldx < K || ldw < K ||
+      (glu && N % 2) || ldo < (glu ? N / 2 : N))
+    return ERR_BAD_ARGUMENT;
+  if (pad != 16 || tiles > 65535 * 16) return ERR_UNSUPPORTED_SIZE;
+  if (tiles > 65535) return ERR_UNSUPPORTED_SIZE;
+  if (dtype == DT_F32 && out_dtype == DT_F32)
+    launch_expert_gemm<float, float>((const float*)x, ldx, x_rows, (const float*)W, expert_stride, ldw, N, K, source,
+                                     tile_expert, tiles, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+  else if (dtype == DT_BF16 && out_dtype == DT_BF16)
+    launch_expert_gemm<bf16_t, bf16_t>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
+                                       tile_expert, tiles, gather, glu, limit, alpha, offset, (bf16_t*)out, ldo, stream);
+  else if (dtype == DT_BF16 && out_dtype == DT_F32)
+    launch_expert_gemm<bf16_t, float>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
+                                      tile_expert, tiles, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// ---------------------------------------------------------------- a token's weighted sum
+template <typename TS>
+__global__ void moe_combine_kernel(const float* __restrict__ down, long ld, const int* __restrict__ place,
+                                   const float* __restrict__ weights, int top, const TS* __restrict__ shared, long shared_ld,
+                                   const float* __restrict__ gate, float* __restrict__ out, int d) {
+  const long token = blockIdx.x;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float total = 0.f;
+    for (int k = 0; k < top; ++k)
+      total = fmaf(weights[token * top + k], down[(long)place[token * top + k] * ld + i], total);
+    if (shared) total = fmaf(gate[token], to_float(shared[token * shared_ld + i]), total);
+    out[token * d + i] = total;
+  }
+}
+
+extern "C" int mi_moe_combine(const float* down, long ld, const int* place, const float* weights, int top,
+                              const void* shared, int shared_dtype, long shared_ld, const float* gate, float* out, int T,
+                              int d, hipStream_t stream) {
+  if (!down || !place || !weights || !out || T <= 0 || d <= 0 || top <= 0 || ld < d || (shared && (!gate || shared_ld < d)))
+    return ERR_BAD_ARGUMENT;
+  if (shared_dtype == DT_F32)
+    moe_combine_kernel<float><<<T, 256, 0, stream>>>(down, ld, place, weights, top, (const float*)shared, shared_ld, gate, out, d);
+  else if (shared_dtype == DT_BF16)
+    moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>(down, ld, place, weights, top, (const bf16_t*)shared, shared_ld, gate, out, d);
+  else
+    return ERR_BAD_ARGUMENT;
+  RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

@@ -62,7 +62,7 @@ _SIGNATURES = {
     },
     "moe": {
         "mi_moe_route": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
-        "mi_moe_plan": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+        "mi_moe_plan": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
         "mi_moe_expert_gemm": [_c_ptr, _c_int, _c_long, _c_int, _c_ptr, _c_long, _c_long, _c_int, _c_int, _c_ptr, _c_ptr,
                                _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_ptr, _c_int, _c_long,
                                _c_ptr],
