@@ -4,7 +4,7 @@ MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|f32] [--layers L]
     python bench.py --workload serving [--shape 0.5b|7b|34b]
     python bench.py --microbench
-    python bench.py --design mukutar [--shape 0.5b|7b] [--layers L] [--window W] [--only mukutar|falcon_h1]
+    python bench.py --design mukutar|lutosun [--shape 0.5b|7b] [--layers L] [--window W] [--only mukutar|lutosun|falcon_h1]
 
 One JSON line: ``value`` = decoded tokens a second at batch 8 with every request at a
 2,048-token context (a step = one decode step of the whole batch: model, greedy sampling,
@@ -30,7 +30,8 @@ distance bias and a sink, generalized delta rule, retention; PolyNorm feed-forwa
 sizes are those of ``--shape``, and beside it the Falcon-H1 shape with the same width, layer count, heads and
 feed-forward width: for both the 2,048-token prompt step and decode steps at batch 1, 8 and 64 behind
 2,048-token contexts, each with its fraction of the peak (prompt: flops; decode: bytes the step has to read).
-The default workload and its line are not touched by it.
+``--design lutosun`` does the same for a Lutosun-shaped model (latent attention, a routed mixture of experts beside
+a shared one, layer norms, a hashed bigram embedding).  The default workload and its line are not touched by either.
 
 ``--workload serving`` runs whole requests through the scheduler and the sampler instead
 (``LLM.generate``): for the 7B shape (and the 0.5B one) 64 requests with prompt lengths uniform in
@@ -148,11 +149,30 @@ def mukutar_shape(shape: dict, layers: int, window: int) -> dict:
             "layers": [dict(kinds[index % 3], mlp=mlp) for index in range(layers)]}
 
 
+def lutosun_shape(shape: dict, layers: int) -> dict:
+    """A Lutosun configuration with the sizes of a Falcon-H1 ``shape``: the same width, vocabulary, heads and head
+    size (half of it more, turned); a key/value latent of two heads' width (as far as the attention kernels' 256
+    dimensions a cached row allow) and a query latent of half the model's width; sixteen experts a quarter as wide as the shape's feed-forward, of which a token uses
+    three beside a shared one of the same width (as many products a token as the dense feed-forward); no looped
+    layers; a bigram table of 16,384 rows."""
+    width, dim, heads = shape["hidden_size"], shape["head_dim"], shape["num_attention_heads"]
+    turned = dim // 2
+    rank = min(2 * dim, 256 - turned)
+    expert = shape["intermediate_size"] // 4
+    mixer = {"heads": heads, "dim": dim, "rot_dim": turned, "vdim": dim, "q_rank": width // 2, "kv_rank": rank,
+             "rot": {"base": 1e6, "dims": turned}, "scale": (dim + turned) ** -0.5}
+    mlp = {"kind": "moe", "expert": {"ff": expert, "limit": 7.0}, "router": {"experts": 16, "top": 3, "scale": 1.0},
+           "shared": {"ff": expert, "limit": 7.0}}
+    return {"architecture": "Lutosun", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
+            "residual_mult": 1.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 16384, "mul_prev": 31, "mul_cur": 17}},
+            "logit_softcap": 30.0, "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
+
+
 def design_points(args) -> int:
-    """Prompt and decode steps of a Mukutar-shaped model and of the Falcon-H1 shape of equal sizes."""
+    """Prompt and decode steps of a model of another design with the sizes of a Falcon-H1 shape, and of that shape."""
     import torch
     from macllm_infer_amd import Engine, Lane
-    from macllm_infer_amd.config import FalconH1Config, MukutarConfig
+    from macllm_infer_amd.config import FalconH1Config, LutosunConfig, MukutarConfig
     from macllm_infer_amd.sampling import GREEDY, Sampler, SamplerRow
     from macllm_infer_amd.weights.random_init import random_tensors
 
@@ -160,8 +180,11 @@ def design_points(args) -> int:
     layers = args.layers or 12
     storage = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     element = 2 if args.dtype == "bf16" else 4
-    configs = {"mukutar": MukutarConfig.from_dict(mukutar_shape(shape, layers, args.window)),
-               "falcon_h1": FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))}
+    if args.design == "lutosun":
+        configs = {"lutosun": LutosunConfig.from_dict(lutosun_shape(shape, layers))}
+    else:
+        configs = {"mukutar": MukutarConfig.from_dict(mukutar_shape(shape, layers, args.window))}
+    configs["falcon_h1"] = FalconH1Config.from_dict(dict(shape, num_hidden_layers=layers))
     batches = [] if args.prefill_only else ([args.batch] if args.skip_points else sorted({1, args.batch, 64}))
     largest = max(batches, default=1)
     per_request = -(-(CONTEXT + args.steps + args.warmup + 1) // 64) * 64
@@ -234,10 +257,10 @@ def design_points(args) -> int:
         out[name] = record
         del engine, sampler
         torch.cuda.empty_cache()
-    first = out.get("mukutar") or next(iter(out.values()))
+    first = out.get(args.design) or next(iter(out.values()))
     headline = first.get(f"decode_b{args.batch}", first["prefill"])
     print(json.dumps({
-        "metric": "Mukutar-shaped model beside the Falcon-H1 shape of equal sizes: prefill tok/s at 2,048 tokens, "
+        "metric": f"{args.design.capitalize()}-shaped model beside the Falcon-H1 shape of equal sizes: prefill tok/s at 2,048 tokens, "
                   "decode tok/s at batch 1 / 8 / 64 behind 2,048-token contexts",
         "value": headline["value"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "higher_is_better": True, "dtype": args.dtype, "data": "synthetic",
@@ -313,11 +336,11 @@ def main() -> int:
                         help="steps: the headline decode and prefill steps; serving: whole requests through the scheduler")
     parser.add_argument("--microbench", action="store_true",
                         help="only this GPU's streaming read and read-modify-write bandwidth")
-    parser.add_argument("--design", default=None, choices=["mukutar"],
+    parser.add_argument("--design", default=None, choices=["mukutar", "lutosun"],
                         help="measure a model of this design with the sizes of --shape (12 layers unless --layers) beside "
                              "the Falcon-H1 shape of equal sizes, instead of the headline workload")
     parser.add_argument("--window", type=int, default=1024, help="--design: the attention layers' window")
-    parser.add_argument("--only", default=None, choices=["mukutar", "falcon_h1"], help="--design: one of the two models")
+    parser.add_argument("--only", default=None, choices=["mukutar", "lutosun", "falcon_h1"], help="--design: one of the two models")
     parser.add_argument("--write-config", default=None, metavar="PATH",
                         help="write the config.json of --shape / --layers there and exit (what "
                              "utils.kernel_trace --config reads)")
@@ -332,6 +355,8 @@ def main() -> int:
         with open(args.write_config, "w") as handle:
             if args.design == "mukutar" and args.only != "falcon_h1":
                 json.dump(mukutar_shape(shape, args.layers or 12, args.window), handle)
+            elif args.design == "lutosun" and args.only != "falcon_h1":
+                json.dump(lutosun_shape(shape, args.layers or 12), handle)
             else:
                 layers = args.layers or (12 if args.design else shape["num_hidden_layers"])
                 json.dump(dict(shape, num_hidden_layers=layers), handle)

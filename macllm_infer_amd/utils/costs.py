@@ -36,7 +36,7 @@ def model_sizes(spec) -> dict:
     d = spec.hidden_size
     total = dict(in_weights=0, out_weights=0, gate_up=0, down=0, kv_per_token=0, state=0, conv_tail=0,
                  attention=0, scan=0, layers=len(spec.schedule), head=spec.vocab_size * d, hidden=d,
-                 mixed=0, inner=0, in_width=0, windows=[], linear_scan=0)
+                 mixed=0, inner=0, in_width=0, windows=[], linear_scan=0, experts=[])
     for entry in spec.schedule:
         layer = spec.layers[entry.layer]
         for slot in layer.mixers:
@@ -53,6 +53,19 @@ def model_sizes(spec) -> dict:
                                          (kv + values) if entry.kv_from is None else 0, part.window))
                 total["mixed"] += mixed
                 total["in_width"] += q + kv + values
+            elif part.kind == "latent_attention":
+                heads, rank, turned = part.num_heads, part.kv_rank, part.rope_dim
+                q = heads * (part.head_dim + turned)
+                # down-projections, the queries' up-projection and their way into the latent space; out of it and out
+                total["in_weights"] += (part.q_rank + rank + turned) * d + q * part.q_rank + heads * part.head_dim * rank
+                total["out_weights"] += heads * part.value_dim * rank + d * heads * part.value_dim
+                cached = (rank + turned) if entry.kv_from is None else 0        # one latent and one turned part a token
+                total["kv_per_token"] += cached
+                # every head scores against the cached row and sums latents: keys rank + turned wide, values rank wide
+                total["attention"] += heads * (2 * rank + turned) / 2.0
+                total["windows"].append((heads * (2 * rank + turned) / 2.0, cached, part.window))
+                total["mixed"] += heads * part.value_dim + heads * rank
+                total["in_width"] += part.q_rank + rank + turned + q + heads * (rank + turned)
             elif part.kind == "retention":
                 keys, values = part.num_heads * part.key_dim, part.num_heads * part.value_dim
                 total["in_weights"] += (2 * keys + 2 * values) * d
@@ -83,6 +96,14 @@ def model_sizes(spec) -> dict:
             total["gate_up"] += 2 * layer.ffn.intermediate_size * d
             total["down"] += d * layer.ffn.intermediate_size
             total["inner"] += layer.ffn.intermediate_size
+        elif layer.ffn.kind == "routed_experts":
+            ffn = layer.ffn
+            shared = ffn.shared_size or 0
+            # what every token uses whatever it chooses: the router, the shared expert and its gate
+            total["gate_up"] += (ffn.num_experts + (1 if shared else 0)) * d + 2 * shared * d
+            total["down"] += d * shared
+            total["inner"] += shared + ffn.top_k * ffn.expert_size
+            total["experts"].append((ffn.num_experts, ffn.top_k, 2 * ffn.expert_size * d, d * ffn.expert_size))
         elif layer.ffn.kind == "polynorm_ffn":
             total["gate_up"] += layer.ffn.intermediate_size * d
             total["down"] += d * layer.ffn.intermediate_size
@@ -97,10 +118,22 @@ def keys_seen(tokens: float, window) -> float:
     return window * (window + 1) / 2.0 + (tokens - window) * window
 
 
+def experts_touched(experts: int, top_k: int, rows: float) -> float:
+    """How many of ``experts`` a step of ``rows`` tokens reads when every token picks ``top_k`` at random."""
+    return experts * (1.0 - (1.0 - top_k / experts) ** rows)
+
+
 def decode_step_costs(spec, batch: int, context: float, element: int = 2) -> Dict[str, Cost]:
-    """A step of ``batch`` single tokens whose requests hold ``context`` tokens each."""
+    """A step of ``batch`` single tokens whose requests hold ``context`` tokens each.  Routed experts: the matrices
+    of as many experts as the step's tokens reach when they choose at random."""
     s = model_sizes(spec)
     rows = batch
+    for experts, top_k, gate_up, down in s["experts"]:
+        touched = experts_touched(experts, top_k, rows)
+        s["gate_up"] += touched * gate_up * 1.0
+        s["down"] += touched * down * 1.0
+    routed_flops = sum(2.0 * rows * top_k * (gate_up + down) - 2.0 * rows * experts_touched(experts, top_k, rows) * (gate_up + down)
+                       for experts, top_k, gate_up, down in s["experts"])
     kept = lambda window: min(context, window) if window else context          # keys a query still sees
     kv_read = sum(per_token * kept(window) for _, per_token, window in s["windows"])
     attention_flops = sum(4.0 * width * kept(window) for width, _, window in s["windows"])
@@ -110,7 +143,8 @@ def decode_step_costs(spec, batch: int, context: float, element: int = 2) -> Dic
                        batch * (s["kv_per_token"] * element + s["state"] * 4 + s["conv_tail"] * element),
                        batch * (attention_flops + 6.0 * s["scan"] + s["linear_scan"])),
         "output projections": Cost(s["out_weights"] * element, 0, 2.0 * rows * s["out_weights"]),
-        "gate and up projections": Cost(s["gate_up"] * element, 0, 2.0 * rows * s["gate_up"]),
+        # (the flops of routed experts: every row times the experts it chose, not times the experts the step read)
+        "gate and up projections": Cost(s["gate_up"] * element, 0, 2.0 * rows * s["gate_up"] + routed_flops),
         "down projections": Cost(s["down"] * element, 0, 2.0 * rows * s["down"]),
         "output head": Cost(s["head"] * element, batch * spec.vocab_size * 4, 2.0 * rows * s["head"]),
     }
@@ -121,9 +155,13 @@ def prefill_costs(spec, tokens: int, element: int = 2) -> Dict[str, Cost]:
     s = model_sizes(spec)
     T = tokens
     weights = s["in_weights"] + s["out_weights"] + s["gate_up"] + s["down"]
+    # routed experts: every matrix is read (a long prompt reaches all of them), a token computes with top_k of them
+    routed_read = sum(experts * (gate_up + down) for experts, _, gate_up, down in s["experts"])
+    routed_flops = sum(2.0 * T * top_k * (gate_up + down) for _, top_k, gate_up, down in s["experts"])
     rows_moved = T * element * (s["hidden"] * 4 * s["layers"] + s["in_width"] + s["mixed"] + 3 * s["inner"])
     return {
-        "matrix products": Cost(weights * element + rows_moved, 0, 2.0 * T * weights + 2.0 * s["head"]),
+        "matrix products": Cost((weights + routed_read) * element + rows_moved, 0,
+                                2.0 * T * weights + routed_flops + 2.0 * s["head"]),
         "attention": Cost(T * s["kv_per_token"] * element, T * s["kv_per_token"] * element,
                           sum(4.0 * width * keys_seen(T, window) for width, _, window in s["windows"])),
         "state-space scan": Cost(s["state"] * 4, s["state"] * 4, 6.0 * s["scan"] * T + s["linear_scan"] * T),
@@ -146,7 +184,7 @@ def total(costs: Dict[str, Cost]) -> Cost:
 DECODE_GROUPS: List[Tuple[str, str]] = [
     (r"mixer_decode_kernel|mixer_merge_kernel|decode_attention_kernel|decode_merge_kernel|ssm_scan_kernel|conv_step_kernel|"
      r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel|paged_attention_tile_kernel|"
-     r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel", "mixers"),
+     r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel|latent_|rotate_heads_kernel", "mixers"),
     (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
     (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
     (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
@@ -154,9 +192,9 @@ DECODE_GROUPS: List[Tuple[str, str]] = [
 ]
 PLAIN_PRODUCT = r"fused_gemm_kernel<\d+, [01], 0"
 PREFILL_GROUPS: List[Tuple[str, str]] = [
-    (r"^Cijk_|gemm_f32_kernel", "matrix products"),
+    (r"^Cijk_|gemm_f32_kernel|head_gemm_kernel|moe_expert_gemm_kernel", "matrix products"),
     (r"prefill_attention|paged_attention_kernel|paged_attention_tile_kernel|paged_attention_merge_kernel|"
-     r"rope_kv_store_kernel", "attention"),
+     r"rope_kv_store_kernel|latent_", "attention"),
     (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel|linear_state_|head_norm_gate_kernel|"
      r"tanh_rows_kernel", "state-space scan"),
 ]

@@ -388,7 +388,9 @@ def test_the_mixture_of_experts_alone(dtype, hidden, experts, top, inner, limit,
         scores = torch.softmax(x.double() @ plain["p.router"].T, dim=-1) + plain["p.correction"]
         ranked = scores.sort(dim=-1, descending=True).values
         clear = (ranked[:, top - 1] - ranked[:, top]) > 2e-2 if top < experts else torch.ones(T, dtype=torch.bool)
-        close(got.cpu()[clear], want[clear], dtype)
+        assert T < 8 or int(clear.sum()) * 2 >= T, "most tokens' choices are clear"
+        if bool(clear.any()):
+            close(got.cpu()[clear], want[clear], dtype)
     else:
         close(got, want, dtype)
 
