@@ -24,11 +24,12 @@ typedef __bf16 mfma_bf16x4 __attribute__((ext_vector_type(4)));
 typedef float mfma_floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned mfma_uintx4 __attribute__((ext_vector_type(4)));
 
-template <int DH, int NSET>
+// DH: the width of a key (and of a query); DV: the width of a value, the keys' unless it is given (a multiple of 16).
+template <int DH, int NSET, int DV = DH>
 struct AttnAccumulator {
   float m[NSET];                       // running maximum of this lane's column in each set, in units of log2 (merge with exp2)
   float l[NSET];                       // this lane's share of the normalizer (summed over q at the end)
-  mfma_floatx4 o[NSET][DH / 16];       // O^T[dims 16*dt + 4q + i][column n]
+  mfma_floatx4 o[NSET][DV / 16];       // O^T[dims 16*dt + 4q + i][column n]
 
   __device__ __forceinline__ void clear() {
 #pragma unroll
@@ -36,7 +37,7 @@ struct AttnAccumulator {
       m[s] = -INFINITY;
       l[s] = 0.f;
 #pragma unroll
-      for (int dt = 0; dt < DH / 16; ++dt) o[s][dt] = mfma_floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int dt = 0; dt < DV / 16; ++dt) o[s][dt] = mfma_floatx4{0.f, 0.f, 0.f, 0.f};
     }
   }
 };
@@ -54,14 +55,14 @@ struct AttnCache {
 // The K and V fragments of STEPS steps of 32 keys from key k00 on.  K: rows of two 16-key tiles
 // per step; V^T: columns of the same 32 keys.  Keys past last_key are clamped to it (their cells
 // are masked or zeroed by attn_compute).
-template <int DH, int STEPS>
+template <int DH, int STEPS, int DV = DH>
 struct AttnFragments {
   mfma_bf16x8 k[STEPS][2][DH / 32];
-  mfma_bf16x8 v[STEPS][DH / 16];
+  mfma_bf16x8 v[STEPS][DV / 16];
 };
 
-template <int DH, int STEPS>
-__device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS>& f, int k00, int last_key, const AttnCache& cache) {
+template <int DH, int STEPS, int DV = DH>
+__device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS, DV>& f, int k00, int last_key, const AttnCache& cache) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int q = lane / 16;
   const int r = lane % 16;
@@ -85,12 +86,12 @@ __device__ __forceinline__ void attn_load(AttnFragments<DH, STEPS>& f, int k00, 
       offset[t] = key % cache.page_size;
     }
 #pragma unroll
-    for (int dt = 0; dt < DH / 16; ++dt) {
+    for (int dt = 0; dt < DV / 16; ++dt) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const mfma_bf16x4 part = *reinterpret_cast<const mfma_bf16x4*>(
             cache.v_base + (long)page[t] * cache.page_stride +
-            ((long)cache.kvh * DH + 16 * dt + r) * cache.page_size + offset[t]);
+            ((long)cache.kvh * DV + 16 * dt + r) * cache.page_size + offset[t]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) f.v[st][dt][4 * t + j] = part[j];
       }
@@ -112,8 +113,8 @@ struct AttnLogBias {
 // MASKED = false: the caller vouches that every key of the round is visible to every column
 // and lies inside the run (steps away from the diagonal, the window's edge and the run's end):
 // no masks are computed.
-template <int DH, int NSET, int STEPS, bool MASKED = true, bool BIASED = false>
-__device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, AttnFragments<DH, STEPS>& f,
+template <int DH, int NSET, int STEPS, bool MASKED = true, bool BIASED = false, int DV = DH>
+__device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET, DV>& acc, AttnFragments<DH, STEPS, DV>& f,
                                              const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                              const int (&col_pos)[NSET], int window, float scale, int k00,
                                              int key_hi, const AttnLogBias<NSET>& bias = AttnLogBias<NSET>()) {
@@ -134,7 +135,7 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
         const unsigned lo = valid >= 2 ? 0xffffffffu : (valid == 1 ? 0x0000ffffu : 0u);
         const unsigned hi = valid >= 4 ? 0xffffffffu : (valid == 3 ? 0x0000ffffu : 0u);
 #pragma unroll
-        for (int dt = 0; dt < DH / 16; ++dt) {
+        for (int dt = 0; dt < DV / 16; ++dt) {
           mfma_uintx4 bits = __builtin_bit_cast(mfma_uintx4, f.v[st][dt]);
           bits[2 * t] &= lo;
           bits[2 * t + 1] &= hi;
@@ -203,7 +204,7 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
         }
       acc.l[s] = acc.l[s] * correction + sum;
 #pragma unroll
-      for (int dt = 0; dt < DH / 16; ++dt) {
+      for (int dt = 0; dt < DV / 16; ++dt) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc.o[s][dt][i] *= correction;
         acc.o[s][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[st][dt], p_frag, acc.o[s][dt], 0, 0, 0);
@@ -221,8 +222,8 @@ __device__ __forceinline__ void attn_compute(AttnAccumulator<DH, NSET>& acc, Att
 // with long runs; a caller whose run is one round of STEPS steps gains nothing from it.
 // min_pos / max_pos: the smallest and largest position among the columns of the wave, when all
 // of them hold queries and the caller knows (the same value in every lane), else -1.
-template <int DH, int NSET, int STEPS, bool PIPELINED = false, bool BIASED = false>
-__device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
+template <int DH, int NSET, int STEPS, bool PIPELINED = false, bool BIASED = false, int DV = DH>
+__device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET, DV>& acc,
                                             const mfma_bf16x8 (&q_frag)[NSET][DH / 32],
                                             const int (&col_pos)[NSET], int window, float scale, int key_lo,
                                             int key_hi, const AttnCache& cache, int min_pos = -1, int max_pos = -1,
@@ -232,13 +233,14 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
   if (PIPELINED) {
     // the next round is always asked for, also past the end of the run (its keys are clamped to
     // the last one and never used): a condition around the loads would cost a wait
-    AttnFragments<DH, STEPS> even, odd;
-    attn_load<DH, STEPS>(even, key_lo, last_key, cache);
+    AttnFragments<DH, STEPS, DV> even, odd;
+    attn_load<DH, STEPS, DV>(even, key_lo, last_key, cache);
     for (int k00 = key_lo; k00 < key_hi; k00 += 2 * ROUND) {
-      attn_load<DH, STEPS>(odd, k00 + ROUND, last_key, cache);
-      attn_compute<DH, NSET, STEPS>(acc, even, q_frag, col_pos, window, scale, k00, key_hi);
-      attn_load<DH, STEPS>(even, k00 + 2 * ROUND, last_key, cache);
-      if (k00 + ROUND < key_hi) attn_compute<DH, NSET, STEPS>(acc, odd, q_frag, col_pos, window, scale, k00 + ROUND, key_hi);
+      attn_load<DH, STEPS, DV>(odd, k00 + ROUND, last_key, cache);
+      attn_compute<DH, NSET, STEPS, true, false, DV>(acc, even, q_frag, col_pos, window, scale, k00, key_hi);
+      attn_load<DH, STEPS, DV>(even, k00 + 2 * ROUND, last_key, cache);
+      if (k00 + ROUND < key_hi)
+        attn_compute<DH, NSET, STEPS, true, false, DV>(acc, odd, q_frag, col_pos, window, scale, k00 + ROUND, key_hi);
     }
   } else {
     // rounds all of whose keys every column of the wave sees run without masks, in a loop of
@@ -247,21 +249,21 @@ __device__ __forceinline__ void attend_keys(AttnAccumulator<DH, NSET>& acc,
     if (min_pos >= 0 && (window <= 0 || key_lo >= max_pos - window + 1))
       open_hi = key_lo + max(0, (min(min_pos + 1, key_hi) - key_lo) / ROUND) * ROUND;
     for (int k00 = key_lo; k00 < open_hi; k00 += ROUND) {
-      AttnFragments<DH, STEPS> f;
-      attn_load<DH, STEPS>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, false, BIASED>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
+      AttnFragments<DH, STEPS, DV> f;
+      attn_load<DH, STEPS, DV>(f, k00, last_key, cache);
+      attn_compute<DH, NSET, STEPS, false, BIASED, DV>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
     }
     for (int k00 = open_hi; k00 < key_hi; k00 += ROUND) {
-      AttnFragments<DH, STEPS> f;
-      attn_load<DH, STEPS>(f, k00, last_key, cache);
-      attn_compute<DH, NSET, STEPS, true, BIASED>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
+      AttnFragments<DH, STEPS, DV> f;
+      attn_load<DH, STEPS, DV>(f, k00, last_key, cache);
+      attn_compute<DH, NSET, STEPS, true, BIASED, DV>(acc, f, q_frag, col_pos, window, scale, k00, key_hi, bias);
     }
   }
 }
 
 // The normalizer of lane's column: the shares of the four lanes (q = 0..3) that hold it.
-template <int DH, int NSET>
-__device__ __forceinline__ float attn_normalizer(const AttnAccumulator<DH, NSET>& acc, int s) {
+template <int DH, int NSET, int DV = DH>
+__device__ __forceinline__ float attn_normalizer(const AttnAccumulator<DH, NSET, DV>& acc, int s) {
   float l = acc.l[s];
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);

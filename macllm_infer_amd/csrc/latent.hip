@@ -222,3 +222,305 @@ extern "C" int mi_head_gemm(const void* x, int dtype, long ldx, long x_col, cons
   RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
+
+// ---------------------------------------------------------------- prompt portions on the matrix cores
+// Attention of a step's prompt portions over the cached rows [latent | turned part] (DK wide, one row a token for
+// all heads; the values are the first DV of them, kept a second time transposed as the V pages), bfloat16.  The
+// queries are already in the latent space.  A workgroup takes 16 consecutive tokens of one lane and NSET heads,
+// which share every key and value fragment; its eight waves split the keys [0, last position] in runs of whole
+// 32-key steps and merge through LDS, set by set (the scheme of the grouped-query prompt kernel, with every head in
+// the one group).  Softmax in float32, in units of log2.
+#include "attn_mfma.h"
+
+#define LATENT_WAVES 8
+
+template <int DK, int DV, int NSET, int STEPS>
+__global__ void __launch_bounds__(LATENT_WAVES * WAVE)
+latent_attention_kernel(const bf16_t* __restrict__ q, long q_ld, int H, const bf16_t* __restrict__ k_base,
+                        const bf16_t* __restrict__ v_base, long page_stride, int page_size,
+                        const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
+                        const int* __restrict__ cu_seqlens, const int* __restrict__ start_pos, float scale, int window,
+                        bf16_t* __restrict__ out, long out_ld) {
+  constexpr int ITEMS = 2 + 4 * (DV / 16);                    // m, l and the accumulator of one set
+  __shared__ float part[LATENT_WAVES][ITEMS][WAVE];
+  __shared__ int wave_pages[LATENT_WAVES][WAVE];
+  // heavy tiles first; every other head pass the other way round
+  const int block = (blockIdx.z & 1) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  const int tile = block / 4;
+  const int head0 = blockIdx.z * NSET;
+  const int request = tiles[2 * tile];
+  if (request < 0) return;                                    // a row of the table past the step's own runs
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wave = threadIdx.x / WAVE;
+  const int qd = lane / 16;
+  const int n = lane % 16;
+  const int lane_end = cu_seqlens[request + 1];
+  const int first_token = tiles[2 * tile + 1] + 16 * (block % 4);
+  if (first_token >= lane_end) return;                        // the whole workgroup
+  const int token = first_token + n;
+  const bool has_query = token < lane_end;
+  const int base_position = start_pos[request] - cu_seqlens[request];
+  const int position = base_position + token;
+  const int last_position = base_position + min(first_token + 15, lane_end - 1);
+  const int first_position = base_position + first_token;
+  const bool full_tile = first_token + 16 <= lane_end && head0 + NSET <= H;
+
+  mfma_bf16x8 q_frag[NSET][DK / 32];
+  int col_pos[NSET];
+#pragma unroll
+  for (int s = 0; s < NSET; ++s) {
+    const bool valid = has_query && head0 + s < H;
+    col_pos[s] = valid ? position : -1;
+#pragma unroll
+    for (int kk = 0; kk < DK / 32; ++kk) {
+      if (valid) {
+        q_frag[s][kk] = *reinterpret_cast<const mfma_bf16x8*>(q + (long)token * q_ld + (long)(head0 + s) * DK +
+                                                               32 * kk + 8 * qd);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q_frag[s][kk][j] = (bf16_t)0.f;
+      }
+    }
+  }
+  AttnAccumulator<DK, NSET, DV> acc;
+  acc.clear();
+  AttnCache cache;
+  cache.k_base = k_base;
+  cache.v_base = v_base;
+  cache.page_stride = page_stride;
+  cache.page_size = page_size;
+  cache.kvh = 0;
+  const int* cache_pages = block_tables + (long)request * max_pages;
+  int key_lo = 0;
+  if (window > 0 && first_position - window + 1 > 0) key_lo = ((first_position - window + 1) / 32) * 32;
+  const int key_hi = last_position + 1;
+  const int steps = (key_hi - key_lo + 31) / 32;
+  const int steps_per_wave = (steps + LATENT_WAVES - 1) / LATENT_WAVES;
+  const int my_lo = key_lo + 32 * steps_per_wave * wave;
+  const int my_hi = min(key_hi, my_lo + 32 * steps_per_wave);
+  // the page ids of the run go through LDS, 64 pages at a time (a wave's own corner of it: no barrier)
+  for (int part_lo = my_lo; part_lo < my_hi;) {
+    const int first_page = part_lo / page_size;
+    const int part_hi = min(my_hi, (first_page + WAVE) * page_size);
+    wave_pages[wave][lane] = cache_pages[min(first_page + lane, max_pages - 1)];
+    cache.pages = wave_pages[wave];
+    cache.base_page = first_page;
+    attend_keys<DK, NSET, STEPS, false, false, DV>(acc, q_frag, col_pos, window, scale, part_lo, part_hi, cache,
+                                                   full_tile ? first_position : -1, last_position);
+    part_lo = part_hi;
+  }
+
+  // merge: set s is finished by wave s
+#pragma unroll
+  for (int s = 0; s < NSET; ++s) {
+    __syncthreads();
+    part[wave][0][lane] = acc.m[s];
+    part[wave][1][lane] = acc.l[s];
+#pragma unroll
+    for (int dt = 0; dt < DV / 16; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[wave][2 + 4 * dt + i][lane] = acc.o[s][dt][i];
+    __syncthreads();
+    if (wave != s % LATENT_WAVES) continue;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < LATENT_WAVES; ++w) m = fmaxf(m, part[w][0][lane]);
+    float factor[LATENT_WAVES];
+    float l = 0.f;
+#pragma unroll
+    for (int w = 0; w < LATENT_WAVES; ++w) {
+      const float m_w = part[w][0][lane];
+      factor[w] = m_w == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_w - m);
+      l += part[w][1][lane] * factor[w];
+    }
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    if (col_pos[s] < 0) continue;
+    const float inverse = 1.f / l;
+    bf16_t* o = out + (long)token * out_ld + (long)(head0 + s) * DV;
+#pragma unroll
+    for (int dt = 0; dt < DV / 16; ++dt) {
+      mfma_bf16x4 packed;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float value = 0.f;
+#pragma unroll
+        for (int w = 0; w < LATENT_WAVES; ++w) value += part[w][2 + 4 * dt + i][lane] * factor[w];
+        packed[i] = (bf16_t)(value * inverse);
+      }
+      *reinterpret_cast<mfma_bf16x4*>(o + 16 * dt + 4 * qd) = packed;
+    }
+  }
+}
+
+// The widths the kernel is built for: (latent, turned part).  most: how many heads share a fragment at most.
+#define LATENT_SHAPES(CASE)                                                                                        \
+  CASE(32, 32, 4, 4) CASE(64, 32, 4, 2) CASE(64, 64, 4, 2) CASE(96, 32, 2, 2) CASE(128, 32, 2, 1) CASE(128, 64, 2, 1) \
+  CASE(192, 64, 1, 1)
+
+extern "C" int mi_latent_attention_supported(int rank, int turned) {
+#define SUPPORTED_CASE(RANK_, TURNED_, MOST_, STEPS_) \
+  if (rank == RANK_ && turned == TURNED_) return 1;
+  LATENT_SHAPES(SUPPORTED_CASE)
+#undef SUPPORTED_CASE
+  return 0;
+}
+
+template <int DK, int DV, int MOST, int STEPS>
+static int launch_latent_attention(const bf16_t* q, long q_ld, int H, const bf16_t* k_base, const bf16_t* v_base,
+                                   long page_stride, int page_size, const int* block_tables, int max_pages,
+                                   const int* tiles, int n_tiles, const int* cu_seqlens, const int* start_pos, float scale,
+                                   int window, bf16_t* out, long out_ld, hipStream_t stream) {
+  const int passes = (H + MOST - 1) / MOST;
+  const int per_pass = (H + passes - 1) / passes;
+  const dim3 grid(4 * n_tiles, 1, passes);
+#define LATENT_LAUNCH(NSET_)                                                                                       \
+  latent_attention_kernel<DK, DV, NSET_, STEPS><<<grid, LATENT_WAVES * WAVE, 0, stream>>>(                         \
+      q, q_ld, H, k_base, v_base, page_stride, page_size, block_tables, max_pages, tiles, cu_seqlens, start_pos, scale, \
+      window, out, out_ld)
+  if (MOST >= 4 && per_pass > 2) LATENT_LAUNCH(MOST >= 4 ? 4 : 1);
+  else if (MOST >= 2 && per_pass > 1) LATENT_LAUNCH(MOST >= 2 ? 2 : 1);
+  else LATENT_LAUNCH(1);
+#undef LATENT_LAUNCH
+  return 0;
+}
+
+// tiles: int32 [n_tiles, 2] = (lane, first token row) of runs of up to 64 tokens of one lane; the step's own keys
+// must be in the cache already.  ERR_UNSUPPORTED_SIZE for widths the kernel is not built for.
+extern "C" int mi_latent_attention(const void* q, long q_ld, int H, int rank, int turned, const void* k_base,
+                                   const void* v_base, long page_stride, int page_size, const int* block_tables,
+                                   int max_pages, const int* tiles, int n_tiles, const int* cu_seqlens,
+                                   const int* start_pos, float scale, int window, void* out, long out_ld,
+                                   hipStream_t stream) {
+  if (!q || !k_base || !v_base || !block_tables || !tiles || !cu_seqlens || !start_pos || !out || n_tiles <= 0 || H <= 0 ||
+      page_size <= 0 || max_pages <= 0)
+    return ERR_BAD_ARGUMENT;
+  if (page_size % 4 != 0 || q_ld % 8 != 0 || out_ld % 4 != 0 || ((unsigned long long)q % 16) != 0 ||
+      ((unsigned long long)out % 8) != 0 || n_tiles > (1 << 28) || H > 65535 * 4)
+    return ERR_UNSUPPORTED_SIZE;
+#define LATENT_CASE(RANK_, TURNED_, MOST_, STEPS_)                                                                 \
+  if (rank == RANK_ && turned == TURNED_) {                                                                        \
+    launch_latent_attention<RANK_ + TURNED_, RANK_, MOST_, STEPS_>(                                                \
+        (const bf16_t*)q, q_ld, H, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, block_tables, \
+        max_pages, tiles, n_tiles, cu_seqlens, start_pos, scale, window, (bf16_t*)out, out_ld, stream);            \
+    RETURN_IF_LAUNCH_FAILED();                                                                                     \
+    return 0;                                                                                                      \
+  }
+  LATENT_SHAPES(LATENT_CASE)
+#undef LATENT_CASE
+  return ERR_UNSUPPORTED_SIZE;
+}
+
+// ---------------------------------------------------------------- single decoded tokens, the context split
+// For steps of single-token lanes in bfloat16: a wave takes one run of `split_keys` keys of one request and up to
+// 16 heads, which are the columns of the matrix cores' products (all heads read the same cached rows, so a key or
+// value fragment is fetched once for the sixteen); it leaves an unnormalized partial result with its maximum and
+// normalizer (in units of log2), and a second kernel merges a token's runs in ascending order.  grid = (runs,
+// tokens, sets of 16 heads), one wave a workgroup.
+template <int DK, int DV, int STEPS>
+__global__ void __launch_bounds__(WAVE)
+latent_decode_kernel(const bf16_t* __restrict__ q, long q_ld, int H, const bf16_t* __restrict__ k_base,
+                     const bf16_t* __restrict__ v_base, long page_stride, int page_size,
+                     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ lane_of_token,
+                     const int* __restrict__ positions, float scale, int window, int split_keys, int splits,
+                     float* __restrict__ partial_o, float* __restrict__ partial_ml) {
+  const int split = blockIdx.x;
+  const long token = blockIdx.y;
+  const int head0 = blockIdx.z * 16;
+  const int pos = positions[token];
+  int first_key = 0;
+  if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
+  const int range_lo = (first_key / 32) * 32 + split * split_keys;
+  if (range_lo > pos) return;                                 // the merge knows which runs hold keys
+  const int range_hi = min(range_lo + split_keys, pos + 1);
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int qd = lane / 16;
+  const int n = lane % 16;
+  const int head = head0 + n;
+  const bool valid = head < H;
+  mfma_bf16x8 q_frag[1][DK / 32];
+  int col_pos[1] = {valid ? pos : -1};
+#pragma unroll
+  for (int kk = 0; kk < DK / 32; ++kk) {
+    if (valid) {
+      q_frag[0][kk] = *reinterpret_cast<const mfma_bf16x8*>(q + token * q_ld + (long)head * DK + 32 * kk + 8 * qd);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q_frag[0][kk][j] = (bf16_t)0.f;
+    }
+  }
+  AttnAccumulator<DK, 1, DV> acc;
+  acc.clear();
+  AttnCache cache;
+  cache.k_base = k_base;
+  cache.v_base = v_base;
+  cache.page_stride = page_stride;
+  cache.page_size = page_size;
+  cache.kvh = 0;
+  cache.pages = block_tables + (long)lane_of_token[token] * max_pages;
+  cache.base_page = 0;
+  attend_keys<DK, 1, STEPS, false, false, DV>(acc, q_frag, col_pos, window, scale, range_lo, range_hi, cache);
+  const float l = attn_normalizer<DK, 1, DV>(acc, 0);
+  if (!valid) return;
+  const long at = (token * H + head) * splits + split;
+  if (qd == 0) {
+    partial_ml[2 * at] = acc.m[0];
+    partial_ml[2 * at + 1] = l;
+  }
+#pragma unroll
+  for (int dt = 0; dt < DV / 16; ++dt)
+    *reinterpret_cast<mfma_floatx4*>(partial_o + at * DV + 16 * dt + 4 * qd) = acc.o[0][dt];
+}
+
+__global__ void latent_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
+                                           const int* __restrict__ positions, int window, int split_keys, int splits,
+                                           int H, int dv, bf16_t* __restrict__ out, long out_ld) {
+  const long token = blockIdx.x;
+  const int head = blockIdx.y;
+  const int pos = positions[token];
+  int first_key = 0;
+  if (window > 0 && pos - window + 1 > 0) first_key = pos - window + 1;
+  const int used = min(splits, (pos - (first_key / 32) * 32) / split_keys + 1);
+  const float* ml = partial_ml + (token * H + head) * splits * 2;
+  const float* o = partial_o + (token * H + head) * (long)splits * dv;
+  float maximum = -INFINITY;
+  for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
+  float denominator = 0.f;
+  for (int s = 0; s < used; ++s)
+    denominator += (ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - maximum)) * ml[2 * s + 1];
+  for (int dim = threadIdx.x; dim < dv; dim += blockDim.x) {
+    float sum = 0.f;
+    for (int s = 0; s < used; ++s)
+      sum += (ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - maximum)) * o[(long)s * dv + dim];
+    out[token * out_ld + (long)head * dv + dim] = (bf16_t)(sum / denominator);
+  }
+}
+
+// partial_o: float32 [T, H, splits, rank]; partial_ml: float32 [T, H, splits, 2].  split_keys: a multiple of 32.
+extern "C" int mi_latent_decode_attention(const void* q, long q_ld, int T, int H, int rank, int turned, const void* k_base,
+                                          const void* v_base, long page_stride, int page_size, const int* block_tables,
+                                          int max_pages, const int* lane_of_token, const int* positions, float scale,
+                                          int window, int split_keys, int splits, float* partial_o, float* partial_ml,
+                                          void* out, long out_ld, hipStream_t stream) {
+  if (!q || !k_base || !v_base || !block_tables || !lane_of_token || !positions || !partial_o || !partial_ml || !out ||
+      T <= 0 || H <= 0 || page_size <= 0 || max_pages <= 0 || splits <= 0 || split_keys <= 0)
+    return ERR_BAD_ARGUMENT;
+  if (page_size % 4 != 0 || q_ld % 8 != 0 || ((unsigned long long)q % 16) != 0 || split_keys % 32 != 0 || T > 65535 ||
+      (H + 15) / 16 > 65535)
+    return ERR_UNSUPPORTED_SIZE;
+  const dim3 grid(splits, T, (H + 15) / 16);
+#define LATENT_DECODE_CASE(RANK_, TURNED_, MOST_, STEPS_)                                                          \
+  if (rank == RANK_ && turned == TURNED_) {                                                                        \
+    latent_decode_kernel<RANK_ + TURNED_, RANK_, (RANK_ + TURNED_ <= 128 ? 2 : 1)><<<grid, WAVE, 0, stream>>>(     \
+        (const bf16_t*)q, q_ld, H, (const bf16_t*)k_base, (const bf16_t*)v_base, page_stride, page_size, block_tables, \
+        max_pages, lane_of_token, positions, scale, window, split_keys, splits, partial_o, partial_ml);            \
+    RETURN_IF_LAUNCH_FAILED();                                                                                     \
+    latent_decode_merge_kernel<<<dim3(T, H), RANK_ <= 64 ? 64 : 128, 0, stream>>>(                                 \
+        partial_o, partial_ml, positions, window, split_keys, splits, H, RANK_, (bf16_t*)out, out_ld);             \
+    RETURN_IF_LAUNCH_FAILED();                                                                                     \
+    return 0;                                                                                                      \
+  }
+  LATENT_SHAPES(LATENT_DECODE_CASE)
+#undef LATENT_DECODE_CASE
+  return ERR_UNSUPPORTED_SIZE;
+}

@@ -156,9 +156,13 @@ extern "C" int mi_moe_plan(const int* chosen, int entries, int top, int E, int p
 }
 
 // ---------------------------------------------------------------- the grouped product
-// Tile t of 16 places belongs to expert tile_expert[t] (none: the workgroup leaves).  GLU: the expert's matrix is
-// [2 I, K], gate rows then up rows; out[place, n] = act(gate tile, up tile), n < I.  Places without a row get zeros.
-template <typename T, typename TO, bool VEC, bool GLU>
+// Tile t of 16 MT places belongs to expert tile_expert[t] (none: the workgroup leaves).  A workgroup owns the
+// tile's rows and PAIRS tiles of 16 output features.  GLU: the expert's matrix is [2 I, K], gate rows then up
+// rows; out[place, n] = act(gate tile, up tile), n < I.  Places without a row get zeros.  Steps of few rows take
+// MT = 1 (every expert's matrix is read once, by as many workgroups as it has tiles of features); prompt portions,
+// whose experts get dozens of rows each, MT = 4 and four tiles of features (the rows and the matrix come from the
+// caches, 64 x 64 results a workgroup).
+template <typename T, typename TO, bool VEC, bool GLU, int MT, int PAIRS>
 __global__ void __launch_bounds__(TILE_THREADS)
 moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride, long ldw,
                        int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert, int gather,
@@ -170,48 +174,56 @@ moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* _
   const int tid = threadIdx.x;
   const int r = (tid & (WAVE - 1)) % 16;
   const int width = GLU ? N / 2 : N;
-  const long n0 = (long)blockIdx.x * 16;
+  const long n0 = (long)blockIdx.x * 16 * PAIRS;
   const T* matrix = W + (long)expert * expert_stride;
-  const long n_row = min(n0 + r, (long)width - 1);
-  const int place_in = tile * 16 + r;
-  const int from = source[place_in];
-  const long x_at = gather ? max(from, 0) : place_in;
-  const T* x_row[1] = {x + min(x_at, (long)x_rows - 1) * ldx};
-  constexpr int NT = GLU ? 2 : 1;
+  constexpr int NT = GLU ? 2 * PAIRS : PAIRS;
   const T* w_row[NT];
-  w_row[0] = matrix + n_row * ldw;
-  if (GLU) w_row[NT - 1] = matrix + (width + n_row) * ldw;
-  tile_floatx4 acc[NT][1];
-  tile_accumulate<T, 1, NT, VEC>(w_row, x_row, K, acc);
-  float value = tile_reduce(acc[0][0], red);
-  if (GLU) {
-    const float up = tile_reduce(acc[NT - 1][0], red);
-    const float g = fminf(value, limit);
-    const float u = fminf(fmaxf(up, -limit), limit);
-    value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+  const T* x_row[MT];
+#pragma unroll
+  for (int p = 0; p < PAIRS; ++p) {
+    const long n_row = min(n0 + 16 * p + r, (long)width - 1);
+    w_row[p] = matrix + n_row * ldw;
+    if (GLU) w_row[NT - PAIRS + p] = matrix + (width + n_row) * ldw;
   }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int place_in = (tile * MT + mt) * 16 + r;
+    const long x_at = gather ? max(source[place_in], 0) : place_in;
+    x_row[mt] = x + min(x_at, (long)x_rows - 1) * ldx;
+  }
+  tile_floatx4 acc[NT][MT];
+  tile_accumulate<T, MT, NT, VEC>(w_row, x_row, K, acc);
   const int l = tid % 64;
-  const long n = n0 + 4 * (l / 16) + tid / 64;
-  const int place = tile * 16 + (l % 16);
-  if (n < width) out[(long)place * ldo + n] = from_float<TO>(source[place] >= 0 ? value : 0.f);
+#pragma unroll
+  for (int p = 0; p < PAIRS; ++p)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float value = tile_reduce(acc[p][mt], red);
+      if (GLU) {
+        const float up = tile_reduce(acc[NT - PAIRS + p][mt], red);
+        const float g = fminf(value, limit);
+        const float u = fminf(fmaxf(up, -limit), limit);
+        value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+      }
+      const long n = n0 + 16 * p + 4 * (l / 16) + tid / 64;
+      const int place = (tile * MT + mt) * 16 + (l % 16);
+      if (n < width) out[(long)place * ldo + n] = from_float<TO>(source[place] >= 0 ? value : 0.f);
+    }
 }
 
 template <typename T, typename TO>
 static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, long expert_stride, long ldw, int N, int K,
-                               const int* source, const int* tile_expert, int tiles, int gather, int glu, float limit,
-                               float alpha, float offset, TO* out, long ldo, hipStream_t stream) {
+                               const int* source, const int* tile_expert, int tiles, int pad, int gather, int glu,
+                               float limit, float alpha, float offset, TO* out, long ldo, hipStream_t stream) {
   constexpr int PIECE = TileTraits<T>::PIECE;
   const bool vec = K % PIECE == 0 && ldx % PIECE == 0 && ldw % PIECE == 0 && expert_stride % PIECE == 0 &&
                    ((unsigned long long)x % 16) == 0 && ((unsigned long long)W % 16) == 0;
   const int width = glu ? N / 2 : N;
-  const dim3 grid((unsigned)((width + 15) / 16), (unsigned)tiles);
-#define EXPERT_LAUNCH(VEC_, GLU_)                                                                                      \
-  moe_expert_gemm_kernel<T, TO, VEC_, GLU_><<<grid, TILE_THREADS, 0, stream>>>(                                       \
-      x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
-  if (vec && glu) EXPERT_LAUNCH(true, true);
-  else if (vec) EXPERT_LAUNCH(true, false);
-  else if (glu) EXPERT_LAUNCH(false, true);
-  else EXPERT_LAUNCH(false, false);
+#define EXPERT_LAUNCH(VEC_, GLU_, MT_, PAIRS_)                                                                           moe_expert_gemm_kernel<T, TO, VEC_, GLU_, MT_, PAIRS_>                                                                    <<<dim3((unsigned)((width + 16 * PAIRS_ - 1) / (16 * PAIRS_)), (unsigned)tiles), TILE_THREADS, 0, stream>>>(               x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
+#define EXPERT_SHAPE(MT_, PAIRS_GLU_, PAIRS_PLAIN_)                                                                      do {                                                                                                                    if (vec && glu) EXPERT_LAUNCH(true, true, MT_, PAIRS_GLU_);                                                            else if (vec) EXPERT_LAUNCH(true, false, MT_, PAIRS_PLAIN_);                                                           else if (glu) EXPERT_LAUNCH(false, true, MT_, PAIRS_GLU_);                                                             else EXPERT_LAUNCH(false, false, MT_, PAIRS_PLAIN_);                                                                 } while (0)
+  if (pad == 64) EXPERT_SHAPE(4, 2, 4);
+  else EXPERT_SHAPE(1, 1, 1);
+#undef EXPERT_SHAPE
 #undef EXPERT_LAUNCH
 }
 
@@ -222,17 +234,16 @@ extern "C" int mi_moe_expert_gemm(const void* x, int dtype, long ldx, int x_rows
   if (!x || !W || !source || !tile_expert || !out || x_rows <= 0 || N <= 0 || K <= 0 || tiles <= 0 || ldx < K || ldw < K ||
       (glu && N % 2) || ldo < (glu ? N / 2 : N))
     return ERR_BAD_ARGUMENT;
-  if (pad != 16 || tiles > 65535 * 16) return ERR_UNSUPPORTED_SIZE;
-  if (tiles > 65535) return ERR_UNSUPPORTED_SIZE;
+  if ((pad != 16 && pad != 64) || tiles > 65535) return ERR_UNSUPPORTED_SIZE;
   if (dtype == DT_F32 && out_dtype == DT_F32)
     launch_expert_gemm<float, float>((const float*)x, ldx, x_rows, (const float*)W, expert_stride, ldw, N, K, source,
-                                     tile_expert, tiles, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+                                     tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
   else if (dtype == DT_BF16 && out_dtype == DT_BF16)
     launch_expert_gemm<bf16_t, bf16_t>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
-                                       tile_expert, tiles, gather, glu, limit, alpha, offset, (bf16_t*)out, ldo, stream);
+                                       tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (bf16_t*)out, ldo, stream);
   else if (dtype == DT_BF16 && out_dtype == DT_F32)
     launch_expert_gemm<bf16_t, float>((const bf16_t*)x, ldx, x_rows, (const bf16_t*)W, expert_stride, ldw, N, K, source,
-                                      tile_expert, tiles, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
+                                      tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();

@@ -59,6 +59,10 @@ _SIGNATURES = {
                          _c_int, _c_int, _c_int, _c_ptr],
         "mi_latent_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int, _c_ptr, _c_int,
                                 _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_ptr, _c_long, _c_ptr],
+        "mi_latent_attention_supported": [_c_int, _c_int],
+        "mi_latent_decode_attention": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_long, _c_int,
+                                       _c_ptr, _c_int, _c_ptr, _c_ptr, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                                       _c_ptr, _c_long, _c_ptr],
     },
     "moe": {
         "mi_moe_route": [_c_ptr, _c_long, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
@@ -533,11 +537,86 @@ def head_linear(x: torch.Tensor, x_col: int, x_head_stride: int, weight: torch.T
 
 def latent_attention_supported(dtype, num_heads: int, kv_rank: int, rope_dim: int, page_size: int) -> bool:
     """Whether the matrix-core kernel for prompt portions of latent attention covers this geometry."""
-    return False
+    return (dtype == torch.bfloat16 and page_size % 4 == 0
+            and bool(_fn("latent", "mi_latent_attention_supported")(int(kv_rank), int(rope_dim))))
+
+
+def latent_attention(q: torch.Tensor, num_heads: int, kv_rank: int, rope_dim: int, k_cache: torch.Tensor,
+                     v_cache: torch.Tensor, block_tables: torch.Tensor, query_tiles: torch.Tensor, cu_seqlens: torch.Tensor,
+                     start_pos: torch.Tensor, scale: float, window: Optional[int], out: torch.Tensor) -> None:
+    """Causal attention of prompt portions over cached latent rows on the matrix cores (bfloat16, online softmax in
+    float32).  ``q`` [T, heads * (kv_rank + rope_dim)]: every head's query in the latent space beside its turned
+    part; K pages [pages, 1, page_size, kv_rank + rope_dim], V pages [pages, 1, kv_rank, page_size];
+    ``query_tiles`` [tiles, 2]: (lane, first token row) of runs of up to 64 tokens of one lane; the step's own rows
+    must be in the cache already.  ``out`` [T, heads * kv_rank]: the attended latents."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    width = kv_rank + rope_dim
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "latent_attention: bfloat16 only")
+    _need(q.shape[1] >= num_heads * width and out.shape == (T, num_heads * kv_rank) and q_ld % 8 == 0
+          and q.data_ptr() % 16 == 0 and out_ld % 4 == 0 and out.data_ptr() % 8 == 0,
+          "latent_attention: q/out shapes or alignment do not fit")
+    page_stride, page_size = _cache_view(k_cache, v_cache, 1, width, q.dtype, kv_rank)
+    _need(latent_attention_supported(q.dtype, num_heads, kv_rank, rope_dim, page_size),
+          "latent_attention: geometry not covered; use paged_attention")
+    for name, tensor in (("block_tables", block_tables), ("query_tiles", query_tiles), ("cu_seqlens", cu_seqlens),
+                         ("start_pos", start_pos)):
+        _i32(tensor, name)
+    _need(block_tables.dim() == 2 and query_tiles.dim() == 2 and query_tiles.shape[1] == 2
+          and cu_seqlens.numel() == start_pos.numel() + 1, "latent_attention: metadata shapes do not match")
+    _check(_fn("latent", "mi_latent_attention")(
+        _p(q), q_ld, num_heads, kv_rank, rope_dim, _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables),
+        block_tables.shape[1], _p(query_tiles), query_tiles.shape[0], _p(cu_seqlens), _p(start_pos), float(scale),
+        int(window or 0), _p(out), out_ld, _stream()), "latent_attention")
+
+
+def latent_decode_attention(q: torch.Tensor, num_heads: int, kv_rank: int, rope_dim: int, k_cache: torch.Tensor,
+                            v_cache: torch.Tensor, block_tables: torch.Tensor, lane_of_token: torch.Tensor,
+                            positions: torch.Tensor, scale: float, window: Optional[int], max_seq_len: int,
+                            out: torch.Tensor) -> None:
+    """``latent_attention`` for steps of single decoded tokens: a request's context is split over many waves, and
+    the heads, which all read the same cached rows, are the columns of the matrix cores' products.
+    ``max_seq_len``: an upper bound of the longest context in the step."""
+    q_ld = _row_major(q, "q")
+    out_ld = _row_major(out, "out")
+    T = q.shape[0]
+    width = kv_rank + rope_dim
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "latent_decode_attention: bfloat16 only")
+    _need(q.shape[1] >= num_heads * width and out.shape == (T, num_heads * kv_rank) and q_ld % 8 == 0
+          and q.data_ptr() % 16 == 0, "latent_decode_attention: q/out shapes or alignment do not fit")
+    page_stride, page_size = _cache_view(k_cache, v_cache, 1, width, q.dtype, kv_rank)
+    _need(latent_attention_supported(q.dtype, num_heads, kv_rank, rope_dim, page_size),
+          "latent_decode_attention: geometry not covered; use paged_attention")
+    _i32(block_tables, "block_tables")
+    _i32(lane_of_token, "lane_of_token")
+    _i32(positions, "positions")
+    _need(block_tables.dim() == 2 and lane_of_token.numel() == T and positions.numel() == T,
+          "latent_decode_attention: metadata shapes do not match")
+    holds = block_tables.shape[1] * page_size
+    span = max(1, min(int(max_seq_len), holds)) if max_seq_len else holds
+    if window:
+        span = min(span, int(window) + 32)
+    split_keys = 64
+    while split_keys < 1024 and T * -(-span // split_keys) > 4096:
+        split_keys *= 2
+    splits = max(1, -(-span // split_keys) + (1 if window else 0))
+    partial_o = torch.empty((T, num_heads, splits, kv_rank), dtype=torch.float32, device=q.device)
+    partial_ml = torch.empty((T, num_heads, splits, 2), dtype=torch.float32, device=q.device)
+    _check(_fn("latent", "mi_latent_decode_attention")(
+        _p(q), q_ld, T, num_heads, kv_rank, rope_dim, _p(k_cache), _p(v_cache), page_stride, page_size, _p(block_tables),
+        block_tables.shape[1], _p(lane_of_token), _p(positions), float(scale), int(window or 0), split_keys, splits,
+        _p(partial_o), _p(partial_ml), _p(out), out_ld, _stream()), "latent_decode_attention")
 
 
 # --------------------------------------------------------------------------- routed experts
-MOE_TILE_ROWS = 16
+MOE_TILE_ROWS = 16          # places of a tile of the grouped products: steps of few rows
+MOE_WIDE_TILE_ROWS = 64     # and steps whose experts get 64 rows or more each on average
+
+
+def moe_tile_rows(tokens: int, top_k: int, num_experts: int) -> int:
+    """The tile of the grouped products for a step: it depends on the step's size alone, never on its tokens."""
+    return MOE_WIDE_TILE_ROWS if tokens * top_k >= MOE_WIDE_TILE_ROWS * num_experts else MOE_TILE_ROWS
 
 
 def moe_route(logits: torch.Tensor, num_experts: int, top_k: int, correction: torch.Tensor, scale: float, eps: float,
@@ -567,9 +646,10 @@ class MoePlan:
     int32 [capacity / pad] = the expert of every tile of ``pad`` places (-1: an unused tile).  Every expert's rows
     start a tile; ``capacity`` depends on the number of tokens alone."""
 
-    def __init__(self, chosen: torch.Tensor, num_experts: int, pad: int = MOE_TILE_ROWS):
+    def __init__(self, chosen: torch.Tensor, num_experts: int, pad: Optional[int] = None):
         _i32(chosen, "chosen")
         tokens, top_k = chosen.shape
+        pad = moe_tile_rows(tokens, top_k, num_experts) if pad is None else int(pad)
         self.pad, self.tokens, self.top_k = pad, tokens, top_k
         self.capacity = -(-(tokens * top_k + num_experts * (pad - 1)) // pad) * pad
         device = chosen.device
@@ -582,8 +662,8 @@ class MoePlan:
                "moe_plan", f"(experts={num_experts})")
 
 
-def moe_plan(chosen: torch.Tensor, num_experts: int) -> MoePlan:
-    return MoePlan(chosen, num_experts)
+def moe_plan(chosen: torch.Tensor, num_experts: int, pad: Optional[int] = None) -> MoePlan:
+    return MoePlan(chosen, num_experts, pad)
 
 
 def moe_expert_gemm(x: torch.Tensor, plan: MoePlan, weight: torch.Tensor, out: torch.Tensor, gather: bool, glu) -> None:

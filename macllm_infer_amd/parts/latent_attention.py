@@ -100,8 +100,13 @@ class LatentAttention(Mixer):
         tiles = {}
         if step.max_query_len > 1 and 0 < getattr(step, "query_tile", 0) < (1 << 20):
             tiles = dict(query_tiles=step.query_tiles, tile_tokens=step.query_tile, cu_seqlens=step.cu_seqlens)
-        if ops.latent_attention_supported(x.dtype, heads, rank, rope, cache.k_cache.shape[2]) and tiles \
-                and step.query_tile == self.query_tile:
+        fast = ops.latent_attention_supported(x.dtype, heads, rank, rope, cache.k_cache.shape[2])
+        if fast and step.max_query_len == 1:
+            # single decoded tokens: the context split over many waves, the heads as the products' columns
+            ops.latent_decode_attention(latent_q, heads, rank, rope, cache.k_cache, cache.v_cache,
+                                        step.block_tables[cache.group], step.lane_of_token, step.positions, spec.scale,
+                                        spec.window, step.max_seq_len, attended)
+        elif fast and tiles and step.query_tile == self.query_tile:
             ops.latent_attention(latent_q, heads, rank, rope, cache.k_cache, cache.v_cache,
                                  step.block_tables[cache.group], step.query_tiles, step.cu_seqlens, step.start_pos,
                                  spec.scale, spec.window, attended)

@@ -56,10 +56,15 @@ class RoutedExperts(FeedForward):
                                     for number in range(experts)]).to(keep).contiguous().to(build.device)
         self.down = torch.stack([get(f"e{number}.down.weight") for number in range(experts)]) \
             .to(keep).contiguous().to(build.device)
-        router = [get("router.weight").to(torch.float32)]
+        # the router's product has float32 sums; a weight stored in bfloat16 beside bfloat16 rows gives exact float32
+        # products on the matrix cores, so it stays as it is stored; any other keeps 32 bits and the float32 kernel
+        stored = {get("router.weight").dtype} | ({get("shared.sg.weight").dtype} if spec.shared_size is not None else set())
+        route_dtype = torch.bfloat16 if (build.dtype == torch.bfloat16 and stored == {torch.bfloat16} and hidden % 8 == 0) \
+            else torch.float32
+        router = [get("router.weight").to(route_dtype)]
         self.shared = spec.shared_size is not None
         if self.shared:
-            router.append(get("shared.sg.weight").to(torch.float32).reshape(1, hidden))
+            router.append(get("shared.sg.weight").to(route_dtype).reshape(1, hidden))
             self.shared_gate_up = Linear([get("shared.gate.weight"), get("shared.up.weight")], [None, None], build)
             self.shared_down = Linear([get("shared.down.weight")], [None], build)
         self.router = torch.cat(router).contiguous().to(build.device)

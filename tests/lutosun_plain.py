@@ -101,8 +101,20 @@ def route(h: torch.Tensor, prefix: str, tensors, router: dict, compute):
     return chosen, weights
 
 
-def mixture(h: torch.Tensor, prefix: str, tensors, mlp: dict, compute) -> torch.Tensor:
+def choice_margin(h: torch.Tensor, prefix: str, tensors, router: dict, compute) -> torch.Tensor:
+    """Per token, how far the last chosen expert's choice score lies above the best one not chosen (infinite when
+    every expert is chosen): a small margin is a choice that rounding may turn."""
+    scores = torch.softmax(h @ tensors[f"{prefix}.router"].to(compute).T, dim=-1)
+    ranked = (scores + tensors[f"{prefix}.correction"].to(compute)).sort(dim=-1, descending=True).values
+    if router["top"] >= router["experts"]:
+        return torch.full((h.shape[0],), float("inf"), dtype=compute)
+    return ranked[:, router["top"] - 1] - ranked[:, router["top"]]
+
+
+def mixture(h: torch.Tensor, prefix: str, tensors, mlp: dict, compute, margins=None) -> torch.Tensor:
     chosen, weights = route(h, prefix, tensors, mlp["router"], compute)
+    if margins is not None:
+        margins.append(choice_margin(h, prefix, tensors, mlp["router"], compute))
     out = torch.zeros_like(h)
     for number in range(mlp["router"]["experts"]):
         rows, places = torch.nonzero(chosen == number, as_tuple=True)
@@ -129,9 +141,10 @@ def run_order(config: dict):
     return order
 
 
-def forward(tokens, tensors, config, compute=torch.float64, streams=None) -> torch.Tensor:
+def forward(tokens, tensors, config, compute=torch.float64, streams=None, margins=None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  ``streams``: a list that receives the residual stream after
-    every run of a layer."""
+    every run of a layer.  ``margins``: a list that receives, for every run of a mixture of experts, each token's
+    ``choice_margin``."""
     eps = config["norm"]["eps"]
     mult = config["residual_mult"]
     x = embedding(tokens, tensors, config, compute)
@@ -148,7 +161,7 @@ def forward(tokens, tensors, config, compute=torch.float64, streams=None) -> tor
         x = x + mult * latent_attention(normed, f"{prefix}.mix", tensors, layer["mixer"], eps, compute)
         if layer.get("mlp") is not None:
             normed = layer_norm(x, tensors[f"{prefix}.norm2"].to(compute), tensors[f"{prefix}.norm2.b"].to(compute), eps)
-            x = x + mult * mixture(normed, f"{prefix}.mlp", tensors, layer["mlp"], compute)
+            x = x + mult * mixture(normed, f"{prefix}.mlp", tensors, layer["mlp"], compute, margins)
         if streams is not None:
             streams.append(x.clone())
     x = layer_norm(x, tensors["final.norm"].to(compute), tensors["final.norm.b"].to(compute), eps)

@@ -439,8 +439,8 @@ class MoePlan:
             cursor += tiles * pad
 
 
-def moe_plan(chosen, num_experts):
-    return MoePlan(chosen, num_experts)
+def moe_plan(chosen, num_experts, pad=None):
+    return MoePlan(chosen, num_experts, pad or 16)
 
 
 def moe_expert_gemm(x, plan, weight, out, gather, glu):

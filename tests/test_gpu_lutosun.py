@@ -150,7 +150,7 @@ def test_one_product_per_head(dtype, T, heads, N, K, x_col, x_stride, out_col, o
     close(got.float(), want.float(), dtype)
 
 
-@pytest.mark.parametrize("T, experts, top", [(1, 5, 2), (37, 12, 3), (300, 70, 8), (9, 3, 3), (64, 130, 1)])
+@pytest.mark.parametrize("T, experts, top", [(1, 5, 2), (37, 12, 3), (300, 70, 8), (9, 3, 3), (64, 130, 1), (700, 6, 2)])
 def test_the_router_and_the_grouping_of_rows_by_expert(T, experts, top):
     logits = rand(T, experts + 1, seed=1) * 2.0
     correction = rand(experts, seed=2) * 0.05
@@ -164,12 +164,13 @@ def test_the_router_and_the_grouping_of_rows_by_expert(T, experts, top):
     close(got_gate, want_gate, torch.float32, "shared gate")
     plan = ops().moe_plan(got_ids, experts)
     source, place, tile_expert = plan.source.cpu(), plan.place.cpu().long(), plan.tile_expert.cpu()
-    assert plan.capacity % 16 == 0 and plan.capacity >= T * top
+    assert plan.pad == (64 if T * top >= 64 * experts else 16)
+    assert plan.capacity % plan.pad == 0 and plan.capacity >= T * top
     flat = got_ids.cpu().reshape(-1)
     assert sorted(place.tolist()) == sorted(set(place.tolist()))                   # every choice has a place of its own
     for entry in range(T * top):
         assert int(source[place[entry]]) == entry // top
-        assert int(tile_expert[place[entry] // 16]) == int(flat[entry])            # in a tile of its expert
+        assert int(tile_expert[place[entry] // plan.pad]) == int(flat[entry])      # in a tile of its expert
     assert int((source >= 0).sum()) == T * top
     used = tile_expert[tile_expert >= 0]
     assert torch.equal(used, used.sort().values)                                   # experts in turn, no tile shared
@@ -177,7 +178,7 @@ def test_the_router_and_the_grouping_of_rows_by_expert(T, experts, top):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T, experts, top, hidden, inner", [(1, 4, 2, 32, 16), (45, 6, 3, 64, 40), (130, 9, 2, 48, 24),
-                                                            (7, 3, 1, 20, 12)])
+                                                            (7, 3, 1, 20, 12), (400, 5, 2, 72, 88), (300, 3, 2, 36, 20)])
 def test_the_grouped_products_and_the_weighted_sum(dtype, T, experts, top, hidden, inner):
     from macllm_infer_amd.config import ClampedGLUSpec
     glu = ClampedGLUSpec(limit=0.9)
@@ -194,7 +195,7 @@ def test_the_grouped_products_and_the_weighted_sum(dtype, T, experts, top, hidde
     ref_ops.moe_expert_gemm(x, host, gate_up, want_inner, True, glu)
     got_inner = torch.empty(plan.capacity, inner, dtype=dtype, device=DEV)
     ops().moe_expert_gemm(x.to(DEV), plan, gate_up.to(DEV), got_inner, gather=True, glu=glu)
-    used = (host.tile_expert >= 0).repeat_interleave(16)                # tiles without an expert are not written
+    used = (host.tile_expert >= 0).repeat_interleave(plan.pad)          # tiles without an expert are not written
     close(got_inner.float().cpu()[used], want_inner.float()[used], dtype, "gate, up and the activation")
     want_down = torch.zeros(plan.capacity, hidden)
     ref_ops.moe_expert_gemm(want_inner, host, down_w, want_down, False, None)
@@ -281,7 +282,11 @@ def feed_every_way(make_harness, x, plain_rows, dtype, beside=None):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, dim, rope, vdim, q_rank, kv_rank, rotary", [
     (3, 16, 8, 12, 20, 24, 8), (2, 32, 16, 32, 64, 40, 12), (1, 24, 32, 8, 8, 56, 32), (4, 64, 32, 64, 48, 96, 32),
-    (5, 12, 0, 20, 16, 16, 0)])
+    (5, 12, 0, 20, 16, 16, 0),
+    # widths the matrix-core prompt kernel is built for (bfloat16): heads that fill a set of columns, leave a part
+    # of one empty, and need a second pass
+    (2, 16, 32, 16, 24, 32, 32), (5, 48, 32, 40, 72, 64, 32), (3, 32, 32, 64, 40, 128, 32), (9, 24, 64, 32, 32, 64, 64),
+    (2, 64, 64, 32, 32, 128, 64), (3, 96, 64, 64, 64, 192, 64)])
 def test_latent_attention_alone(dtype, heads, dim, rope, vdim, q_rank, kv_rank, rotary):
     hidden, T = 56, 170
     spec = latent_spec(heads, dim, rope, vdim, q_rank, kv_rank, rotary, base=300.0)
@@ -296,15 +301,21 @@ def test_latent_attention_alone(dtype, heads, dim, rope, vdim, q_rank, kv_rank, 
                    beside=rand(40, hidden, seed=3))
 
 
-def far_key_case(distance, T=700, hidden=32):
+def far_key_case(distance, T=700, hidden=32, matrix=False):
     """Inputs and weights of a latent attention layer in which the key ``distance`` tokens behind the last query
     stands out: the turned key part is a plain product of the token's row (no norm), so a row thirty times as large
     gives a key part thirty times as large, and its sign is chosen so that the last query's score for it is the
     largest by far.  Returns (spec, tensors, x, the plain rows, how much of the last row that key accounts for)."""
-    spec = latent_spec(2, 16, 8, 16, 16, 16, 8, base=50.0, scale=1.0)
-    tensors = latent_tensors(hidden, spec, 50)
+    if matrix:          # widths the matrix-core kernels are built for, weights and rows as bfloat16 holds them
+        spec = latent_spec(3, 16, 32, 16, 16, 32, 32, base=50.0, scale=0.5)
+        tensors = rounded(latent_tensors(hidden, spec, 50), torch.bfloat16)
+    else:
+        spec = latent_spec(2, 16, 8, 16, 16, 16, 8, base=50.0, scale=1.0)
+        tensors = latent_tensors(hidden, spec, 50)
     names = {k: v.double() for k, v in plain_names(tensors, "p").items()}
     base = rand(T, hidden, seed=4) * 0.3
+    if matrix:
+        base = base.to(torch.bfloat16).float()
     target = T - 1 - distance
     best = None
     for sign in (1.0, -1.0):
@@ -320,17 +331,20 @@ def far_key_case(distance, T=700, hidden=32):
     return best
 
 
+@pytest.mark.parametrize("matrix", [False, True])
 @pytest.mark.parametrize("feed", ["whole", "decoded", "cut"])
-@pytest.mark.parametrize("distance", [1, 15, 16, 17, 299, 640])
-def test_a_far_key_that_stands_out_is_found(distance, feed):
+@pytest.mark.parametrize("distance", [1, 15, 16, 17, 31, 32, 63, 64, 65, 299, 640])
+def test_a_far_key_that_stands_out_is_found(distance, feed, matrix):
     """Among hundreds of keys one, ``distance`` tokens behind the last query, carries most of the last row's weight.
     With pages of 16 tokens that key lies next to the query, at page borders and far away; it is found from a prompt,
-    from a decoded token, and from a portion cut right behind the key."""
-    spec, tensors, x, want, share = far_key_case(distance)
+    from a decoded token, and from a portion cut right behind the key; by the general kernels in float32 and by the
+    matrix-core kernels in bfloat16 (whose waves split the keys in runs of 32 and 64)."""
+    spec, tensors, x, want, share = far_key_case(distance, matrix=matrix)
     assert share > 0.3, "the crafted key does not stand out"
     T, hidden = x.shape
     target = T - 1 - distance
-    harness = PartHarness(spec, tensors, hidden, torch.float32, page_size=16, capacity=720)
+    dtype = torch.bfloat16 if matrix else torch.float32
+    harness = PartHarness(spec, tensors, hidden, dtype, page_size=16, capacity=720)
     if feed == "whole":
         out, = harness.run([("r", x)])
         got = out[-1]
@@ -340,7 +354,7 @@ def test_a_far_key_that_stands_out_is_found(distance, feed):
     else:
         harness.run([("r", x[:target + 1])])
         got = harness.run([("r", x[target + 1:])])[0][-1]
-    close(got, want[-1], torch.float32, f"distance {distance}")
+    close(got, want[-1], dtype, f"distance {distance}")
 
 
 def experts_spec(experts, top, inner, limit, scale, shared=None):
@@ -416,11 +430,47 @@ def tokens_for(raw, count, seed):
     return torch.randint(0, raw["vocab"], (count,), generator=torch.Generator().manual_seed(seed)).tolist()
 
 
+CLEAR_MARGIN = 0.01
+
+
+class Rows(torch.Tensor):
+    """The plain model's logits with, per position, whether every choice of experts at that position was clear (no
+    expert within ``CLEAR_MARGIN`` of the last chosen one, in any layer): 16-bit rounding may turn a choice that is
+    not, and the logits of that position are then another model's.  Slices keep the flags."""
+
+    @staticmethod
+    def of(logits, clear):
+        rows = logits.as_subclass(Rows)
+        rows.clear = clear
+        return rows
+
+    def __getitem__(self, index):
+        return Rows.of(torch.Tensor.__getitem__(self.as_subclass(torch.Tensor), index), self.clear[index])
+
+
 def plain(raw, tensors, tokens):
-    return lutosun_plain.forward(tokens, tensors, raw).to(torch.float32)
+    margins = []
+    logits = lutosun_plain.forward(tokens, tensors, raw, margins=margins).to(torch.float32)
+    clear = torch.ones(len(tokens), dtype=torch.bool)
+    for margin in margins:
+        clear &= margin > CLEAR_MARGIN
+    return Rows.of(logits, clear)
+
+
+def cat(pieces):
+    return Rows.of(torch.cat([piece.as_subclass(torch.Tensor) for piece in pieces]),
+                   torch.cat([piece.clear.reshape(-1) for piece in pieces]))
 
 
 def same(got, want, dtype, what):
+    clear = getattr(want, "clear", None)
+    want = want.as_subclass(torch.Tensor) if isinstance(want, Rows) else want
+    if dtype != "float32" and clear is not None:
+        clear = clear.reshape(-1)
+        assert want.shape[0] < 20 or int(clear.sum()) * 2 >= want.shape[0], f"{what}: most positions' choices are clear"
+        if not bool(clear.any()):
+            return
+        got, want = got.float().cpu()[clear], want[clear]
     got, want = got.float().cpu().numpy(), want.float().numpy()
     if dtype == "float32":
         error = np.abs(got - want).max(axis=-1)
@@ -460,8 +510,8 @@ def test_whole_cut_decoded_and_mixed_steps_match_the_plain_model(tmp_path, name,
     three = engine.step([Lane("c", first[21:22], [0]), Lane("e", third[140:141], [0]), Lane("d", second[30:41], [10])])
     four = engine.step([Lane("e", third[141:150], [8]), Lane("c", first[22:170], [147])])
     got = torch.cat([one, two, three, four])
-    rows = torch.cat([want[0][19:20], want[1][:3], want[2][0:1], want[2][139:140], want[1][3:30], want[0][20:21],
-                      want[0][21:22], want[2][140:141], want[1][40:41], want[2][149:150], want[0][169:170]])
+    rows = cat([want[0][19:20], want[1][:3], want[2][0:1], want[2][139:140], want[1][3:30], want[0][20:21],
+                want[0][21:22], want[2][140:141], want[1][40:41], want[2][149:150], want[0][169:170]])
     same(got, rows, dtype, "mixed steps")
     engine.cache.check()
 
