@@ -211,6 +211,107 @@ moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* _
     }
 }
 
+// The same product for prompt portions whose rows and matrices are whole 16-byte pieces: a workgroup owns a tile
+// of 64 places and 128 rows of its expert's matrix (GLU: 64 gate rows and the 64 up rows that go with them, which
+// make 64 outputs; else 128 outputs), walks K one chunk at a time through two LDS stages (the next chunk's pieces
+// are asked for before the current one's products), and every wave owns all 64 places and a quarter of the
+// features: no sum crosses a wave, a row's result is summed in k order by one lane's accumulator.
+template <typename T, typename TO, bool GLU>
+__global__ void __launch_bounds__(TILE_THREADS)
+moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride,
+                            long ldw, int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert,
+                            int gather, float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+  typedef typename TileTraits<T>::Piece Piece;
+  constexpr int CHUNK = TileTraits<T>::CHUNK;
+  constexpr int PIECE = TileTraits<T>::PIECE;
+  constexpr int ROWS = 64, FEATURES = 128;
+  __shared__ Piece stage[2][(ROWS + FEATURES) * 4];
+  const int tile = blockIdx.y;
+  const int expert = tile_expert[tile];
+  if (expert < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int q = lane / 16;
+  const int r = lane % 16;
+  const int width = GLU ? N / 2 : N;
+  const long n0 = (long)blockIdx.x * (GLU ? 64 : 128);
+  const T* matrix = W + (long)expert * expert_stride;
+  // what this thread brings into a stage: piece `part` of one row of x and of two rows of the matrix
+  const int lrow = tid / 4;
+  const int part = tid % 4;
+  const int place_in = tile * ROWS + lrow;
+  const long x_at = gather ? max(source[place_in], 0) : place_in;
+  const T* x_from = x + min(x_at, (long)x_rows - 1) * ldx;
+  const T* w_from[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int s = lrow + 64 * j;                                // row of the stage's matrix part
+    long feature;
+    if (GLU) feature = (j == 0 ? 0 : width) + min(n0 + lrow, (long)width - 1);
+    else feature = min(n0 + s, (long)width - 1);
+    w_from[j] = matrix + feature * ldw;
+  }
+  tile_floatx4 acc[2][4];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = tile_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int chunks = (K + CHUNK - 1) / CHUNK;
+  Piece gx = tile_load<T, true>(x_from, PIECE * part, K);
+  Piece gw0 = tile_load<T, true>(w_from[0], PIECE * part, K);
+  Piece gw1 = tile_load<T, true>(w_from[1], PIECE * part, K);
+  stage[0][lrow * 4 + part] = gx;
+  stage[0][(ROWS + lrow) * 4 + part] = gw0;
+  stage[0][(ROWS + 64 + lrow) * 4 + part] = gw1;
+  __syncthreads();
+  for (int c = 0; c < chunks; ++c) {
+    const int cur = c & 1;
+    const int k_next = c + 1 < chunks ? (c + 1) * CHUNK + PIECE * part : K;      // past the end: zeros, never used
+    gx = tile_load<T, true>(x_from, k_next, K);
+    gw0 = tile_load<T, true>(w_from[0], k_next, K);
+    gw1 = tile_load<T, true>(w_from[1], k_next, K);
+    Piece a[2], b[4];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int row = GLU ? 64 * nt + 16 * wave + r : 32 * wave + 16 * nt + r;
+      a[nt] = stage[cur][(ROWS + row) * 4 + q];
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) b[mt] = stage[cur][(16 * mt + r) * 4 + q];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = tile_mfma(a[nt], b[mt], acc[nt][mt]);
+    stage[cur ^ 1][lrow * 4 + part] = gx;
+    stage[cur ^ 1][(ROWS + lrow) * 4 + part] = gw0;
+    stage[cur ^ 1][(ROWS + 64 + lrow) * 4 + part] = gw1;
+    __syncthreads();
+  }
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int place = tile * ROWS + 16 * mt + r;
+    const bool live = source[place] >= 0;
+    TO* row = out + (long)place * ldo;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (GLU) {
+        const long n = n0 + 16 * wave + 4 * q + i;
+        const float g = fminf(acc[0][mt][i], limit);
+        const float u = fminf(fmaxf(acc[1][mt][i], -limit), limit);
+        const float value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+        if (n < width) row[n] = from_float<TO>(live ? value : 0.f);
+      } else {
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+          const long n = n0 + 32 * wave + 16 * nt + 4 * q + i;
+          if (n < width) row[n] = from_float<TO>(live ? acc[nt][mt][i] : 0.f);
+        }
+      }
+    }
+  }
+}
+
 template <typename T, typename TO>
 static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, long expert_stride, long ldw, int N, int K,
                                const int* source, const int* tile_expert, int tiles, int pad, int gather, int glu,
@@ -221,8 +322,19 @@ static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, lon
   const int width = glu ? N / 2 : N;
 #define EXPERT_LAUNCH(VEC_, GLU_, MT_, PAIRS_)                                                                           moe_expert_gemm_kernel<T, TO, VEC_, GLU_, MT_, PAIRS_>                                                                    <<<dim3((unsigned)((width + 16 * PAIRS_ - 1) / (16 * PAIRS_)), (unsigned)tiles), TILE_THREADS, 0, stream>>>(               x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
 #define EXPERT_SHAPE(MT_, PAIRS_GLU_, PAIRS_PLAIN_)                                                                      do {                                                                                                                    if (vec && glu) EXPERT_LAUNCH(true, true, MT_, PAIRS_GLU_);                                                            else if (vec) EXPERT_LAUNCH(true, false, MT_, PAIRS_PLAIN_);                                                           else if (glu) EXPERT_LAUNCH(false, true, MT_, PAIRS_GLU_);                                                             else EXPERT_LAUNCH(false, false, MT_, PAIRS_PLAIN_);                                                                 } while (0)
-  if (pad == 64) EXPERT_SHAPE(4, 2, 4);
-  else EXPERT_SHAPE(1, 1, 1);
+  if (pad == 64 && vec) {
+    const dim3 grid((unsigned)((width + (glu ? 64 : 128) - 1) / (glu ? 64 : 128)), (unsigned)tiles);
+    if (glu)
+      moe_expert_gemm_wide_kernel<T, TO, true><<<grid, TILE_THREADS, 0, stream>>>(
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+    else
+      moe_expert_gemm_wide_kernel<T, TO, false><<<grid, TILE_THREADS, 0, stream>>>(
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+  } else if (pad == 64) {
+    EXPERT_SHAPE(4, 2, 4);
+  } else {
+    EXPERT_SHAPE(1, 1, 1);
+  }
 #undef EXPERT_SHAPE
 #undef EXPERT_LAUNCH
 }
