@@ -472,9 +472,13 @@ latent_decode_kernel(const bf16_t* __restrict__ q, long q_ld, int H, const bf16_
     *reinterpret_cast<mfma_floatx4*>(partial_o + at * DV + 16 * dt + 4 * qd) = acc.o[0][dt];
 }
 
+#define LATENT_MERGE_SPLITS 256
+
 __global__ void latent_decode_merge_kernel(const float* __restrict__ partial_o, const float* __restrict__ partial_ml,
                                            const int* __restrict__ positions, int window, int split_keys, int splits,
                                            int H, int dv, bf16_t* __restrict__ out, long out_ld) {
+  __shared__ float factor[LATENT_MERGE_SPLITS];      // exp2(maximum of the run - maximum), 0 for a run without keys
+  __shared__ float scratch[16];
   const long token = blockIdx.x;
   const int head = blockIdx.y;
   const int pos = positions[token];
@@ -484,14 +488,22 @@ __global__ void latent_decode_merge_kernel(const float* __restrict__ partial_o, 
   const float* ml = partial_ml + (token * H + head) * splits * 2;
   const float* o = partial_o + (token * H + head) * (long)splits * dv;
   float maximum = -INFINITY;
-  for (int s = 0; s < used; ++s) maximum = fmaxf(maximum, ml[2 * s]);
-  float denominator = 0.f;
-  for (int s = 0; s < used; ++s)
-    denominator += (ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - maximum)) * ml[2 * s + 1];
+  for (int s = threadIdx.x; s < used; s += blockDim.x) maximum = fmaxf(maximum, ml[2 * s]);
+  maximum = wave_max(maximum);
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE] = maximum;
+  __syncthreads();
+  for (int w = 0; w < (int)(blockDim.x + WAVE - 1) / WAVE; ++w) maximum = fmaxf(maximum, scratch[w]);
+  float share = 0.f;
+  for (int s = threadIdx.x; s < used; s += blockDim.x) {
+    const float f = ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - maximum);
+    factor[s] = f;
+    share += f * ml[2 * s + 1];
+  }
+  const float denominator = block_sum(share, scratch);           // (its barriers also publish the factors)
   for (int dim = threadIdx.x; dim < dv; dim += blockDim.x) {
     float sum = 0.f;
-    for (int s = 0; s < used; ++s)
-      sum += (ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - maximum)) * o[(long)s * dv + dim];
+    for (int s = 0; s < used; ++s) sum = fmaf(factor[s], o[(long)s * dv + dim], sum);
     out[token * out_ld + (long)head * dv + dim] = (bf16_t)(sum / denominator);
   }
 }
@@ -506,7 +518,7 @@ extern "C" int mi_latent_decode_attention(const void* q, long q_ld, int T, int H
       T <= 0 || H <= 0 || page_size <= 0 || max_pages <= 0 || splits <= 0 || split_keys <= 0)
     return ERR_BAD_ARGUMENT;
   if (page_size % 4 != 0 || q_ld % 8 != 0 || ((unsigned long long)q % 16) != 0 || split_keys % 32 != 0 || T > 65535 ||
-      (H + 15) / 16 > 65535)
+      (H + 15) / 16 > 65535 || H > 65535 || splits > LATENT_MERGE_SPLITS)
     return ERR_UNSUPPORTED_SIZE;
   const dim3 grid(splits, T, (H + 15) / 16);
 #define LATENT_DECODE_CASE(RANK_, TURNED_, MOST_, STEPS_)                                                          \

@@ -368,7 +368,7 @@ __global__ void moe_combine_kernel(const float* __restrict__ down, long ld, cons
                                    const float* __restrict__ weights, int top, const TS* __restrict__ shared, long shared_ld,
                                    const float* __restrict__ gate, float* __restrict__ out, int d) {
   const long token = blockIdx.x;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += gridDim.y * blockDim.x) {
     float total = 0.f;
     for (int k = 0; k < top; ++k)
       total = fmaf(weights[token * top + k], down[(long)place[token * top + k] * ld + i], total);
@@ -382,10 +382,12 @@ extern "C" int mi_moe_combine(const float* down, long ld, const int* place, cons
                               int d, hipStream_t stream) {
   if (!down || !place || !weights || !out || T <= 0 || d <= 0 || top <= 0 || ld < d || (shared && (!gate || shared_ld < d)))
     return ERR_BAD_ARGUMENT;
+  // a step of few tokens spreads a token's features over several workgroups
+  const dim3 grid((unsigned)T, (unsigned)(T >= 256 ? 1 : min((d + 255) / 256, 16)));
   if (shared_dtype == DT_F32)
-    moe_combine_kernel<float><<<T, 256, 0, stream>>>(down, ld, place, weights, top, (const float*)shared, shared_ld, gate, out, d);
+    moe_combine_kernel<float><<<grid, 256, 0, stream>>>(down, ld, place, weights, top, (const float*)shared, shared_ld, gate, out, d);
   else if (shared_dtype == DT_BF16)
-    moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>(down, ld, place, weights, top, (const bf16_t*)shared, shared_ld, gate, out, d);
+    moe_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(down, ld, place, weights, top, (const bf16_t*)shared, shared_ld, gate, out, d);
   else
     return ERR_BAD_ARGUMENT;
   RETURN_IF_LAUNCH_FAILED();

@@ -597,8 +597,9 @@ def latent_decode_attention(q: torch.Tensor, num_heads: int, kv_rank: int, rope_
     span = max(1, min(int(max_seq_len), holds)) if max_seq_len else holds
     if window:
         span = min(span, int(window) + 32)
+    # runs of 64 keys while that leaves the step a few thousand waves, longer ones beyond; at most 256 runs a request
     split_keys = 64
-    while split_keys < 1024 and T * -(-span // split_keys) > 4096:
+    while (split_keys < 1024 and T * -(-span // split_keys) > 4096) or -(-span // split_keys) + 1 > 256:
         split_keys *= 2
     splits = max(1, -(-span // split_keys) + (1 if window else 0))
     partial_o = torch.empty((T, num_heads, splits, kv_rank), dtype=torch.float32, device=q.device)

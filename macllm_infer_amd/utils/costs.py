@@ -186,13 +186,13 @@ DECODE_GROUPS: List[Tuple[str, str]] = [
      r"gate_norm_kernel|rope_kv_store_kernel|paged_attention_kernel|paged_attention_tile_kernel|"
      r"paged_attention_merge_kernel|linear_state_|head_norm_gate_kernel|tanh_rows_kernel|latent_|rotate_heads_kernel", "mixers"),
     (r"fused_gemm_kernel<\d+, \d+, 2|shared_rows_gemm_kernel<\d+, \d+, 2", "input projections"),
-    (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1", "gate and up projections"),
+    (r"fused_gemm_kernel<\d+, \d+, 1|shared_rows_gemm_kernel<\d+, \d+, 1|moe_|clamped_glu_kernel", "gate and up projections"),
     (r"fused_gemm_kernel<\d+, \d+, 3|fused_gemm_kernel<\d+, 2, 0|shared_rows_gemm_kernel<\d+, \d+, 0|fused_gemm_split_kernel",
      "output projections + down projections"),
 ]
 PLAIN_PRODUCT = r"fused_gemm_kernel<\d+, [01], 0"
 PREFILL_GROUPS: List[Tuple[str, str]] = [
-    (r"^Cijk_|gemm_f32_kernel|head_gemm_kernel|moe_expert_gemm_kernel", "matrix products"),
+    (r"^Cijk_|gemm_f32_kernel|head_gemm_kernel|moe_expert_gemm", "matrix products"),
     (r"prefill_attention|paged_attention_kernel|paged_attention_tile_kernel|paged_attention_merge_kernel|"
      r"rope_kv_store_kernel|latent_", "attention"),
     (r"ssd_|ssm_scan_kernel|conv1d_silu|conv_state_update|gate_norm_kernel|linear_state_|head_norm_gate_kernel|"

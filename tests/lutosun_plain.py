@@ -34,6 +34,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor, base: float, dims: int) -> torch.Tensor:
     """x [T, ..., D]: the first ``dims`` dimensions in pairs (2i, 2i + 1) turned by position * base^(-2i/dims)."""
     out = x.clone()
+    if dims == 0:
+        return out
     half = dims // 2
     frequency = torch.tensor([base ** (-2.0 * i / dims) for i in range(half)], dtype=x.dtype)
     angle = positions.to(x.dtype).reshape(-1, *([1] * (x.dim() - 1))) * frequency
@@ -68,7 +70,8 @@ def latent_attention(h: torch.Tensor, prefix: str, tensors, mixer: dict, eps: fl
     tokens = h.shape[0]
     heads, dim, rot_dim, vdim, rank = mixer["heads"], mixer["dim"], mixer["rot_dim"], mixer["vdim"], mixer["kv_rank"]
     positions = torch.arange(tokens)
-    base, rot_dims = mixer["rot"]["base"], mixer["rot"]["dims"]
+    rot = mixer.get("rot") or {"base": 1.0, "dims": 0}
+    base, rot_dims = rot["base"], rot["dims"]
     query_latent = rms_norm(h @ get("dq").T, get("dq.norm"), eps)
     q = (query_latent @ get("uq").T).reshape(tokens, heads, dim + rot_dim)
     q_plain, q_turned = q[..., :dim], rotate_interleaved(q[..., dim:], positions, base, rot_dims)

@@ -595,3 +595,67 @@ def test_greedy_generation_through_the_entry_point(tmp_path, name):
             logits = plain(raw, tensors, prompt + want[:place])[-1]
             top = torch.topk(logits, 2).values
             assert float(top[0] - top[1]) < 1e-3, f"prompt of {len(prompt)}: token {place} differs without a tie"
+
+
+def drawn_configuration(seed):
+    """A configuration with every size and option drawn at random: odd widths and vocabularies, 1 to 7 heads, plain
+    widths that are and are not whole 16-byte pieces, turned parts turned wholly and partly, layers in any number with
+    and without a feed-forward, experts with and without a shared one, any loop, with and without bigram and cap."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *values: values[int(rng.integers(len(values)))]
+    width = int(pick(40, 56, 72, 100, 128, 136))
+    count = int(rng.integers(1, 5))
+    kinds = []
+    for _ in range(int(rng.integers(1, 3))):
+        rot_dim = int(pick(0, 4, 8, 16, 32))
+        mixer = lutosun_configs.latent(int(rng.integers(1, 8)), int(pick(8, 12, 16, 24, 32, 40)), rot_dim,
+                                       int(pick(8, 12, 16, 32, 48)), int(pick(8, 20, 32, 48)), int(pick(8, 16, 24, 32, 64)),
+                                       rot_dims=None if rot_dim < 8 or rng.random() < 0.5 else rot_dim // 2,
+                                       base=float(pick(100.0, 10000.0, 1e6)))
+        experts = int(rng.integers(1, 10))
+        mlp = None
+        if rng.random() < 0.85:
+            mlp = lutosun_configs.moe(experts, int(rng.integers(1, experts + 1)), int(pick(8, 12, 24, 40, 64)),
+                                      float(pick(0.5, 1.0, 3.0)), float(pick(1.0, 1.5, 2.5)),
+                                      shared=None if rng.random() < 0.3 else (int(pick(8, 20, 32, 72)), float(pick(0.5, 1.0, 7.0))))
+        kinds.append(lutosun_configs.with_mlp(mixer, mlp))
+    raw = {"architecture": "Lutosun", "width": width, "vocab": int(pick(61, 97, 256, 301)),
+           "norm": {"eps": float(pick(1e-5, 1e-6))}, "residual_mult": float(pick(0.25, 0.5, 1.0, 1.4)),
+           "embedding": {"scale": float(pick(1.0, 4.0, 12.0))},
+           "layers": [kinds[int(rng.integers(len(kinds)))] for _ in range(count)]}
+    if rng.random() < 0.7:
+        raw["embedding"]["bigram"] = {"buckets": int(pick(1, 7, 64, 509)), "mul_prev": int(pick(1, 31, 1000003)),
+                                      "mul_cur": int(pick(1, 17, 999983))}
+    if rng.random() < 0.7:
+        start = int(rng.integers(0, count))
+        raw["loop"] = {"start": start, "stop": int(rng.integers(start + 1, count + 1)), "times": int(rng.integers(1, 4))}
+    if rng.random() < 0.6:
+        raw["logit_softcap"] = float(pick(5.0, 15.0, 30.0))
+    return raw
+
+
+@pytest.mark.parametrize("seed", list(range(4100, 4116)))
+def test_randomly_drawn_configurations_whole_cut_and_side_by_side(tmp_path, seed):
+    from macllm_infer_amd.engine import Engine, Lane
+    raw, tensors = lutosun_configs.make_model_dir(drawn_configuration(seed), tmp_path, seed=seed, storage_dtype=torch.float32)
+    engine = Engine(str(tmp_path), dtype="float32", device=DEV, kv_cache_block_tokens=int(np.random.default_rng(seed).choice([4, 8, 16])),
+                    kv_cache_capacity_tokens=512, max_active_sequences=3)
+    first, second = tokens_for(raw, 83, seed), tokens_for(raw, 21, seed + 1)
+    want_first, want_second = plain(raw, tensors, first), plain(raw, tensors, second)
+    engine.add_request("whole")
+    same(engine.step([Lane("whole", first, list(range(83)))]), want_first, "float32", f"seed {seed}, whole")
+    engine.finish("whole")
+    engine.add_request("a")
+    engine.add_request("b")
+    rows_a, rows_b, at_a, at_b = [], [], 0, 0
+    for size_a, size_b in ((5, 1), (2, 1), (40, 3), (1, 1), (1, 15), (34, 0)):
+        lanes = [Lane("a", first[at_a:at_a + size_a], list(range(size_a)))]
+        if size_b:
+            lanes.append(Lane("b", second[at_b:at_b + size_b], list(range(size_b))))
+        rows = engine.step(lanes)
+        rows_a.append(rows[:size_a])
+        rows_b.append(rows[size_a:])
+        at_a, at_b = at_a + size_a, at_b + size_b
+    same(torch.cat(rows_a), want_first, "float32", f"seed {seed}, portions beside another request")
+    same(torch.cat(rows_b), want_second, "float32", f"seed {seed}, the other request")
+    engine.cache.check()
