@@ -160,11 +160,11 @@ def lutosun_shape(shape: dict, layers: int) -> dict:
     rank = min(2 * dim, 256 - turned)
     expert = shape["intermediate_size"] // 4
     mixer = {"heads": heads, "dim": dim, "rot_dim": turned, "vdim": dim, "q_rank": width // 2, "kv_rank": rank,
-             "rot": {"base": 1e6, "dims": turned}, "scale": (dim + turned) ** -0.5}
+             "rot": {"base": 5e5, "dims": turned}, "scale": (dim + turned) ** -0.5}
     mlp = {"kind": "moe", "expert": {"ff": expert, "limit": 7.0}, "router": {"experts": 16, "top": 3, "scale": 1.0},
            "shared": {"ff": expert, "limit": 7.0}}
     return {"architecture": "Lutosun", "width": width, "vocab": shape["vocab_size"], "norm": {"eps": 1e-5},
-            "residual_mult": 1.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 16384, "mul_prev": 31, "mul_cur": 17}},
+            "residual_mult": 1.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 16384, "mul_prev": 7919, "mul_cur": 104729}},
             "logit_softcap": 30.0, "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
 
 

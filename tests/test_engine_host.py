@@ -301,6 +301,7 @@ def test_the_limits_are_the_ones_in_the_kernel_sources():
     with open(os.path.join(build.CSRC, "common.hip")) as handle:
         assert "(size_t)d * sizeof(float) > 64 * 1024" in handle.read()
     assert limits.NORM_MAX_WIDTH * 4 == 64 * 1024
+    assert limits.MOE_MAX_EXPERTS == define("moe", "MOE_MAX_EXPERTS")
     # and the sizes at the limits are accepted
     raw = dict(tiny_configs.TINY_B, mamba_d_conv=16, mamba_d_state=512, head_dim=256)
     from macllm_infer_amd.config import FalconH1Config

@@ -81,6 +81,17 @@ def test_a_broken_configuration_names_its_key(broken, text):
         config_from_dict(raw)
 
 
+def test_sizes_that_no_kernel_takes_are_refused_at_load_with_their_key():
+    raw = json.loads(json.dumps(lutosun_configs.LUT_A))
+    raw["layers"][1]["mixer"].update(kv_rank=250, rot_dim=8)              # a cached row of 258 numbers
+    with pytest.raises(ConfigError, match=r"kv_rank \+ rot_dim.*258"):
+        Engine(config=raw, tensors=None, dtype="float32", device="cpu", check_device=False)
+    raw = json.loads(json.dumps(lutosun_configs.LUT_A))
+    raw["layers"][0]["mlp"]["router"]["experts"] = 1025
+    with pytest.raises(ConfigError, match=r"router.experts.*1025"):
+        Engine(config=raw, tensors=None, dtype="float32", device="cpu", check_device=False)
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_whole_cut_and_token_by_token_match_the_plain_model(host_ops, tmp_path, name):
     engine, raw, tensors = engine_for(name, tmp_path)
