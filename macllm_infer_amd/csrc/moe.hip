@@ -26,9 +26,11 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
   if (token >= T) return;
   const float* row = logits + (long)token * ld;
   float score[MOE_PER_LANE], choice[MOE_PER_LANE];
+  const int held = (E + WAVE - 1) / WAVE;          // experts a lane holds: the loops below end there (the same in every lane)
   float most = -INFINITY;
 #pragma unroll
   for (int j = 0; j < MOE_PER_LANE; ++j) {
+    if (j >= held) break;
     const int e = lane + WAVE * j;
     score[j] = e < E ? row[e] : -INFINITY;
     most = fmaxf(most, score[j]);
@@ -37,6 +39,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
   float total = 0.f;
 #pragma unroll
   for (int j = 0; j < MOE_PER_LANE; ++j) {
+    if (j >= held) break;
     const int e = lane + WAVE * j;
     score[j] = e < E ? expf(score[j] - most) : 0.f;
     total += score[j];
@@ -44,6 +47,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
   total = wave_sum(total);
 #pragma unroll
   for (int j = 0; j < MOE_PER_LANE; ++j) {
+    if (j >= held) break;
     const int e = lane + WAVE * j;
     score[j] = score[j] / total;
     choice[j] = e < E ? score[j] + correction[e] : -INFINITY;
@@ -56,6 +60,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
     int best_id = 0x7fffffff;
 #pragma unroll
     for (int j = 0; j < MOE_PER_LANE; ++j) {
+      if (j >= held) break;
       const int e = lane + WAVE * j;
       if (e < E && (choice[j] > best || (choice[j] == best && e < best_id))) {
         best = choice[j];
@@ -76,7 +81,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int T, int E, int to
     }
 #pragma unroll
     for (int j = 0; j < MOE_PER_LANE; ++j)
-      if (lane + WAVE * j == best_id) choice[j] = -INFINITY;
+      if (j < held && lane + WAVE * j == best_id) choice[j] = -INFINITY;
     picked_sum += best_score;
     if ((k & (WAVE - 1)) == lane) {
       // more choices than lanes: written as they come
