@@ -634,16 +634,20 @@ def drawn_configuration(seed):
     return raw
 
 
-@pytest.mark.parametrize("seed", list(range(4100, 4116)))
-def test_randomly_drawn_configurations_whole_cut_and_side_by_side(tmp_path, seed):
+DRAWN = [(seed, "float32") for seed in range(4100, 4116)] + [(seed, "bfloat16") for seed in range(4200, 4212)]
+
+
+@pytest.mark.parametrize("seed, dtype", DRAWN)
+def test_randomly_drawn_configurations_whole_cut_and_side_by_side(tmp_path, seed, dtype):
     from macllm_infer_amd.engine import Engine, Lane
-    raw, tensors = lutosun_configs.make_model_dir(drawn_configuration(seed), tmp_path, seed=seed, storage_dtype=torch.float32)
-    engine = Engine(str(tmp_path), dtype="float32", device=DEV, kv_cache_block_tokens=int(np.random.default_rng(seed).choice([4, 8, 16])),
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    raw, tensors = lutosun_configs.make_model_dir(drawn_configuration(seed), tmp_path, seed=seed, storage_dtype=storage)
+    engine = Engine(str(tmp_path), dtype=dtype, device=DEV, kv_cache_block_tokens=int(np.random.default_rng(seed).choice([4, 8, 16])),
                     kv_cache_capacity_tokens=512, max_active_sequences=3)
     first, second = tokens_for(raw, 83, seed), tokens_for(raw, 21, seed + 1)
     want_first, want_second = plain(raw, tensors, first), plain(raw, tensors, second)
     engine.add_request("whole")
-    same(engine.step([Lane("whole", first, list(range(83)))]), want_first, "float32", f"seed {seed}, whole")
+    same(engine.step([Lane("whole", first, list(range(83)))]), want_first, dtype, f"seed {seed}, whole")
     engine.finish("whole")
     engine.add_request("a")
     engine.add_request("b")
@@ -656,6 +660,6 @@ def test_randomly_drawn_configurations_whole_cut_and_side_by_side(tmp_path, seed
         rows_a.append(rows[:size_a])
         rows_b.append(rows[size_a:])
         at_a, at_b = at_a + size_a, at_b + size_b
-    same(torch.cat(rows_a), want_first, "float32", f"seed {seed}, portions beside another request")
-    same(torch.cat(rows_b), want_second, "float32", f"seed {seed}, the other request")
+    same(torch.cat(rows_a), want_first, dtype, f"seed {seed}, portions beside another request")
+    same(torch.cat(rows_b), want_second, dtype, f"seed {seed}, the other request")
     engine.cache.check()
