@@ -216,6 +216,11 @@ moe_expert_gemm_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* _
     }
 }
 
+// Where piece `piece` (0..3) of row `row` of an LDS stage lies: a row is 64 bytes, and the pieces of rows 4 apart
+// are swapped among themselves so that the sixteen rows a quarter of a wave reads at once fall into sixteen
+// different groups of banks.
+__device__ __forceinline__ int stage_slot(int row, int piece) { return row * 4 + (piece ^ ((row >> 2) & 3)); }
+
 // The same product for prompt portions whose rows and matrices are whole 16-byte pieces: a workgroup owns a tile
 // of 64 places and 128 rows of its expert's matrix (GLU: 64 gate rows and the 64 up rows that go with them, which
 // make 64 outputs; else 128 outputs), walks K one chunk at a time through two LDS stages (the next chunk's pieces
@@ -266,9 +271,9 @@ moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const
   Piece gx = tile_load<T, true>(x_from, PIECE * part, K);
   Piece gw0 = tile_load<T, true>(w_from[0], PIECE * part, K);
   Piece gw1 = tile_load<T, true>(w_from[1], PIECE * part, K);
-  stage[0][lrow * 4 + part] = gx;
-  stage[0][(ROWS + lrow) * 4 + part] = gw0;
-  stage[0][(ROWS + 64 + lrow) * 4 + part] = gw1;
+  stage[0][stage_slot(lrow, part)] = gx;
+  stage[0][stage_slot(ROWS + lrow, part)] = gw0;
+  stage[0][stage_slot(ROWS + 64 + lrow, part)] = gw1;
   __syncthreads();
   for (int c = 0; c < chunks; ++c) {
     const int cur = c & 1;
@@ -280,17 +285,17 @@ moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
       const int row = GLU ? 64 * nt + 16 * wave + r : 32 * wave + 16 * nt + r;
-      a[nt] = stage[cur][(ROWS + row) * 4 + q];
+      a[nt] = stage[cur][stage_slot(ROWS + row, q)];
     }
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) b[mt] = stage[cur][(16 * mt + r) * 4 + q];
+    for (int mt = 0; mt < 4; ++mt) b[mt] = stage[cur][stage_slot(16 * mt + r, q)];
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = tile_mfma(a[nt], b[mt], acc[nt][mt]);
-    stage[cur ^ 1][lrow * 4 + part] = gx;
-    stage[cur ^ 1][(ROWS + lrow) * 4 + part] = gw0;
-    stage[cur ^ 1][(ROWS + 64 + lrow) * 4 + part] = gw1;
+    stage[cur ^ 1][stage_slot(lrow, part)] = gx;
+    stage[cur ^ 1][stage_slot(ROWS + lrow, part)] = gw0;
+    stage[cur ^ 1][stage_slot(ROWS + 64 + lrow, part)] = gw1;
     __syncthreads();
   }
 #pragma unroll
@@ -317,6 +322,116 @@ moe_expert_gemm_wide_kernel(const T* __restrict__ x, long ldx, int x_rows, const
   }
 }
 
+// The widest form, for prompt portions whose experts get hundreds of rows each: 128 places x 128 matrix rows a
+// workgroup, every wave a quarter of it as 64 places x 64 matrix rows (GLU: 32 gate rows and their 32 up rows), so
+// that eight fragments from LDS feed sixteen matrix instructions.
+template <typename T, typename TO, bool GLU>
+__global__ void __launch_bounds__(TILE_THREADS)
+moe_expert_gemm_widest_kernel(const T* __restrict__ x, long ldx, int x_rows, const T* __restrict__ W, long expert_stride,
+                              long ldw, int N, int K, const int* __restrict__ source, const int* __restrict__ tile_expert,
+                              int gather, float limit, float alpha, float offset, TO* __restrict__ out, long ldo) {
+  typedef typename TileTraits<T>::Piece Piece;
+  constexpr int CHUNK = TileTraits<T>::CHUNK;
+  constexpr int PIECE = TileTraits<T>::PIECE;
+  constexpr int ROWS = 128, FEATURES = 128;
+  __shared__ Piece stage[2][(ROWS + FEATURES) * 4];
+  const int tile = blockIdx.y;
+  const int expert = tile_expert[tile];
+  if (expert < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  const int wm = wave / 2;                                     // which 64 places
+  const int wn = wave % 2;                                     // which half of the features
+  const int q = lane / 16;
+  const int r = lane % 16;
+  const int width = GLU ? N / 2 : N;
+  const long n0 = (long)blockIdx.x * (GLU ? 64 : 128);
+  const T* matrix = W + (long)expert * expert_stride;
+  const int lrow = tid / 4;
+  const int part = tid % 4;
+  const T* x_from[2];
+  const T* w_from[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int place_in = tile * ROWS + lrow + 64 * j;
+    const long x_at = gather ? max(source[place_in], 0) : place_in;
+    x_from[j] = x + min(x_at, (long)x_rows - 1) * ldx;
+    long feature;
+    if (GLU) feature = (j == 0 ? 0 : width) + min(n0 + lrow, (long)width - 1);
+    else feature = min(n0 + lrow + 64 * j, (long)width - 1);
+    w_from[j] = matrix + feature * ldw;
+  }
+  tile_floatx4 acc[4][4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = tile_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int chunks = (K + CHUNK - 1) / CHUNK;
+  Piece gx[2], gw[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    gx[j] = tile_load<T, true>(x_from[j], PIECE * part, K);
+    gw[j] = tile_load<T, true>(w_from[j], PIECE * part, K);
+    stage[0][stage_slot(lrow + 64 * j, part)] = gx[j];
+    stage[0][stage_slot(ROWS + lrow + 64 * j, part)] = gw[j];
+  }
+  __syncthreads();
+  for (int c = 0; c < chunks; ++c) {
+    const int cur = c & 1;
+    const int k_next = c + 1 < chunks ? (c + 1) * CHUNK + PIECE * part : K;      // past the end: zeros, never used
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      gx[j] = tile_load<T, true>(x_from[j], k_next, K);
+      gw[j] = tile_load<T, true>(w_from[j], k_next, K);
+    }
+    Piece a[4], b[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      // GLU: nt 0, 1 are gate rows, nt 2, 3 the up rows of the same outputs (the stage's second 64 rows)
+      const int row = GLU ? 64 * (nt / 2) + 32 * wn + 16 * (nt % 2) + r : 64 * wn + 16 * nt + r;
+      a[nt] = stage[cur][stage_slot(ROWS + row, q)];
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) b[mt] = stage[cur][stage_slot(64 * wm + 16 * mt + r, q)];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = tile_mfma(a[nt], b[mt], acc[nt][mt]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      stage[cur ^ 1][stage_slot(lrow + 64 * j, part)] = gx[j];
+      stage[cur ^ 1][stage_slot(ROWS + lrow + 64 * j, part)] = gw[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int place = tile * ROWS + 64 * wm + 16 * mt + r;
+    const bool live = source[place] >= 0;
+    TO* row = out + (long)place * ldo;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (GLU) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const long n = n0 + 32 * wn + 16 * h + 4 * q + i;
+          const float g = fminf(acc[h][mt][i], limit);
+          const float u = fminf(fmaxf(acc[2 + h][mt][i], -limit), limit);
+          const float value = g / (1.0f + expf(-alpha * g)) * (u + offset);
+          if (n < width) row[n] = from_float<TO>(live ? value : 0.f);
+        }
+      } else {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+          const long n = n0 + 64 * wn + 16 * nt + 4 * q + i;
+          if (n < width) row[n] = from_float<TO>(live ? acc[nt][mt][i] : 0.f);
+        }
+      }
+    }
+  }
+}
+
 template <typename T, typename TO>
 static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, long expert_stride, long ldw, int N, int K,
                                const int* source, const int* tile_expert, int tiles, int pad, int gather, int glu,
@@ -327,7 +442,15 @@ static void launch_expert_gemm(const T* x, long ldx, int x_rows, const T* W, lon
   const int width = glu ? N / 2 : N;
 #define EXPERT_LAUNCH(VEC_, GLU_, MT_, PAIRS_)                                                                           moe_expert_gemm_kernel<T, TO, VEC_, GLU_, MT_, PAIRS_>                                                                    <<<dim3((unsigned)((width + 16 * PAIRS_ - 1) / (16 * PAIRS_)), (unsigned)tiles), TILE_THREADS, 0, stream>>>(               x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo)
 #define EXPERT_SHAPE(MT_, PAIRS_GLU_, PAIRS_PLAIN_)                                                                      do {                                                                                                                    if (vec && glu) EXPERT_LAUNCH(true, true, MT_, PAIRS_GLU_);                                                            else if (vec) EXPERT_LAUNCH(true, false, MT_, PAIRS_PLAIN_);                                                           else if (glu) EXPERT_LAUNCH(false, true, MT_, PAIRS_GLU_);                                                             else EXPERT_LAUNCH(false, false, MT_, PAIRS_PLAIN_);                                                                 } while (0)
-  if (pad == 64 && vec) {
+  if (pad == 128) {      // (only plans of rows and matrices in whole pieces are made so wide)
+    const dim3 grid((unsigned)((width + (glu ? 64 : 128) - 1) / (glu ? 64 : 128)), (unsigned)tiles);
+    if (glu)
+      moe_expert_gemm_widest_kernel<T, TO, true><<<grid, TILE_THREADS, 0, stream>>>(
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+    else
+      moe_expert_gemm_widest_kernel<T, TO, false><<<grid, TILE_THREADS, 0, stream>>>(
+          x, ldx, x_rows, W, expert_stride, ldw, N, K, source, tile_expert, gather, limit, alpha, offset, out, ldo);
+  } else if (pad == 64 && vec) {
     const dim3 grid((unsigned)((width + (glu ? 64 : 128) - 1) / (glu ? 64 : 128)), (unsigned)tiles);
     if (glu)
       moe_expert_gemm_wide_kernel<T, TO, true><<<grid, TILE_THREADS, 0, stream>>>(
@@ -351,7 +474,13 @@ extern "C" int mi_moe_expert_gemm(const void* x, int dtype, long ldx, int x_rows
   if (!x || !W || !source || !tile_expert || !out || x_rows <= 0 || N <= 0 || K <= 0 || tiles <= 0 || ldx < K || ldw < K ||
       (glu && N % 2) || ldo < (glu ? N / 2 : N))
     return ERR_BAD_ARGUMENT;
-  if ((pad != 16 && pad != 64) || tiles > 65535) return ERR_UNSUPPORTED_SIZE;
+  if ((pad != 16 && pad != 64 && pad != 128) || tiles > 65535) return ERR_UNSUPPORTED_SIZE;
+  if (pad == 128) {
+    const long piece = dtype == DT_F32 ? 4 : 8;
+    if (K % piece || ldx % piece || ldw % piece || expert_stride % piece || ((unsigned long long)x % 16) ||
+        ((unsigned long long)W % 16))
+      return ERR_UNSUPPORTED_SIZE;
+  }
   if (dtype == DT_F32 && out_dtype == DT_F32)
     launch_expert_gemm<float, float>((const float*)x, ldx, x_rows, (const float*)W, expert_stride, ldw, N, K, source,
                                      tile_expert, tiles, pad, gather, glu, limit, alpha, offset, (float*)out, ldo, stream);

@@ -612,11 +612,14 @@ def latent_decode_attention(q: torch.Tensor, num_heads: int, kv_rank: int, rope_
 
 # --------------------------------------------------------------------------- routed experts
 MOE_TILE_ROWS = 16          # places of a tile of the grouped products: steps of few rows
-MOE_WIDE_TILE_ROWS = 64     # and steps whose experts get 64 rows or more each on average
+MOE_WIDE_TILE_ROWS = 64     # steps whose experts get 64 rows or more each on average
+MOE_WIDEST_TILE_ROWS = 128  # and 256 or more, if rows and matrices are whole 16-byte pieces (``whole_pieces``)
 
 
-def moe_tile_rows(tokens: int, top_k: int, num_experts: int) -> int:
+def moe_tile_rows(tokens: int, top_k: int, num_experts: int, whole_pieces: bool = False) -> int:
     """The tile of the grouped products for a step: it depends on the step's size alone, never on its tokens."""
+    if whole_pieces and tokens * top_k >= 2 * MOE_WIDEST_TILE_ROWS * num_experts:
+        return MOE_WIDEST_TILE_ROWS
     return MOE_WIDE_TILE_ROWS if tokens * top_k >= MOE_WIDE_TILE_ROWS * num_experts else MOE_TILE_ROWS
 
 

@@ -69,6 +69,9 @@ class RoutedExperts(FeedForward):
             self.shared_down = Linear([get("shared.down.weight")], [None], build)
         self.router = torch.cat(router).contiguous().to(build.device)
         self.correction = get("correction").to(torch.float32).contiguous().to(build.device)
+        # rows and matrices in whole 16-byte pieces: the widest tiles of the grouped products take nothing else
+        piece = 4 if keep == torch.float32 else 8
+        self.whole_pieces = hidden % piece == 0 and inner % piece == 0
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         spec = self.spec
@@ -76,7 +79,8 @@ class RoutedExperts(FeedForward):
         logits = ops.linear(x, self.router, None, keep_float32=True)          # float32 [T, experts (+ 1)]
         chosen, weights, gate = ops.moe_route(logits, spec.num_experts, spec.top_k, self.correction, spec.route_scale,
                                               spec.weight_eps, self.shared)
-        plan = ops.moe_plan(chosen, spec.num_experts)
+        plan = ops.moe_plan(chosen, spec.num_experts,
+                            ops.moe_tile_rows(tokens, spec.top_k, spec.num_experts, self.whole_pieces))
         rows = x if x.dtype == self.gate_up.dtype else x.to(self.gate_up.dtype)
         inner = torch.empty((plan.capacity, spec.expert_size), dtype=rows.dtype, device=x.device)
         ops.moe_expert_gemm(rows, plan, self.gate_up, inner, gather=True, glu=spec.activation)

@@ -177,9 +177,10 @@ def test_the_router_and_the_grouping_of_rows_by_expert(T, experts, top):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T, experts, top, hidden, inner", [(1, 4, 2, 32, 16), (45, 6, 3, 64, 40), (130, 9, 2, 48, 24),
-                                                            (7, 3, 1, 20, 12), (400, 5, 2, 72, 88), (300, 3, 2, 36, 20)])
-def test_the_grouped_products_and_the_weighted_sum(dtype, T, experts, top, hidden, inner):
+@pytest.mark.parametrize("T, experts, top, hidden, inner, pad", [
+    (1, 4, 2, 32, 16, None), (45, 6, 3, 64, 40, None), (130, 9, 2, 48, 24, None), (7, 3, 1, 20, 12, None),
+    (400, 5, 2, 72, 88, None), (300, 3, 2, 36, 20, None), (700, 3, 2, 64, 40, 128), (530, 2, 2, 136, 264, 128)])
+def test_the_grouped_products_and_the_weighted_sum(dtype, T, experts, top, hidden, inner, pad):
     from macllm_infer_amd.config import ClampedGLUSpec
     glu = ClampedGLUSpec(limit=0.9)
     x = rand(T, hidden, seed=1).to(dtype)
@@ -187,7 +188,7 @@ def test_the_grouped_products_and_the_weighted_sum(dtype, T, experts, top, hidde
     down_w = (rand(experts, hidden, inner, seed=3) / inner ** 0.5).to(dtype)
     chosen = torch.stack([torch.randperm(experts, generator=torch.Generator().manual_seed(10 + t))[:top] for t in range(T)])
     weights = torch.rand(T, top, generator=torch.Generator().manual_seed(4))
-    plan = ops().moe_plan(chosen.to(torch.int32).to(DEV), experts)
+    plan = ops().moe_plan(chosen.to(torch.int32).to(DEV), experts, pad)          # (pad: the widest tiles, by hand)
     host = ref_ops.MoePlan.__new__(ref_ops.MoePlan)
     host.pad, host.tokens, host.top_k, host.capacity = plan.pad, T, top, plan.capacity
     host.source, host.place, host.tile_expert = plan.source.cpu(), plan.place.cpu(), plan.tile_expert.cpu()
